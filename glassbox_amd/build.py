@@ -46,6 +46,8 @@ LIBRARIES: Dict[str, tuple] = {
     "attention_plain": ("hip", ["hip/attention_plain.hip"], ["hip/common.h"]),
     "attention_bf16": ("hip", ["hip/attention_bf16.hip"], ["hip/common.h", "hip/attention_bf16.h"]),
     "sampling": ("hip", ["hip/sampling.hip"], ["hip/common.h"]),
+    "streams": ("hip", ["hip/streams.hip"], ["hip/common.h"]),
+    "linear_attention": ("hip", ["hip/linear_attention.hip"], ["hip/common.h"]),
 }
 
 _lock = threading.Lock()

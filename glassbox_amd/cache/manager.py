@@ -24,10 +24,12 @@ class CacheError(RuntimeError):
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """One pool of pages: ``kind`` FULL keeps every key, WINDOW only the last ``window``."""
+    """One pool of pages: ``kind`` FULL keeps every key, WINDOW only the last ``window`` and, with ``keep_first``, the
+    first so many for as long as the request lives.  (The order of the fields is that of earlier callers.)"""
     kind: int = FULL
     window: int = 0
     num_pages: int = 0
+    keep_first: int = 0
 
 
 _lib = None
@@ -39,7 +41,7 @@ def _host():
         lib = build.load("host")
         i32p, i64 = C.POINTER(C.c_int32), C.c_int64
         lib.gbh_cache_create.restype = C.c_void_p
-        lib.gbh_cache_create.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+        lib.gbh_cache_create.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
                                          C.POINTER(C.c_int), C.c_int, C.c_int]
         lib.gbh_cache_destroy.argtypes = [C.c_void_p]
         lib.gbh_cache_destroy.restype = None
@@ -88,6 +90,8 @@ class CacheManager:
         for g in groups:
             if g.kind == WINDOW and g.window <= 0:
                 raise CacheError("a window group needs a positive window")
+            if g.keep_first < 0 or (g.keep_first and g.kind != WINDOW):
+                raise CacheError("kept first keys go with a window group")
             if g.num_pages <= 0:
                 raise CacheError("every page group needs at least one page")
         self._lib = _host()
@@ -97,7 +101,7 @@ class CacheManager:
         n = len(groups)
         mk = lambda vals: (C.c_int * max(1, n))(*vals)
         self._h = C.c_void_p(self._lib.gbh_cache_create(
-            page_size, n, mk([g.kind for g in groups]), mk([g.window for g in groups]),
+            page_size, n, mk([g.kind for g in groups]), mk([g.window for g in groups]), mk([g.keep_first for g in groups]),
             mk([g.num_pages for g in groups]), num_state_slots, 1 if share_prefixes else 0))
         self._table_buf = (C.c_int32 * 64)()
         self._copies_buf = (C.c_int32 * (3 * 64))()

@@ -119,6 +119,8 @@ def architecture_of(raw: Dict[str, Any]) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, list) and archs:
         return str(archs[0])
+    if isinstance(raw.get("architecture"), str):   # some configurations name the one architecture plainly
+        return raw["architecture"]
     mt = raw.get("model_type")
     _register_builtin()
     if mt in _MODEL_TYPES:

@@ -92,6 +92,24 @@ __device__ __forceinline__ float key_dot(const float* qs, const T* kb, int slot,
 struct Shape {
   int nh, nkv, hd, page_size, window, table_stride;
   float scale;
+  int keep;   // with a window: keys 0 .. keep - 1 stay visible to every later token
+};
+
+// The chunks of the token at position pos.  Without kept first keys: from lo = the window's first key (or 0) on.
+// With them, where the window has moved past key 0: first the chunks of keys 0 .. min(keep, lo) - 1, then the
+// window's; keys that are both kept and inside the window belong to the window's chunks.
+struct Chunks {
+  int lo, kept, n_kept, n;
+  __device__ __forceinline__ Chunks(const Shape& sh, int pos) {
+    lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
+    kept = sh.keep > 0 ? min(sh.keep, lo) : 0;
+    n_kept = (kept + kChunk - 1) / kChunk;
+    n = n_kept + (pos - lo) / kChunk + 1;
+  }
+  __device__ __forceinline__ int first(int c) const { return c < n_kept ? c * kChunk : lo + (c - n_kept) * kChunk; }
+  __device__ __forceinline__ int last(int c, int pos) const {
+    return c < n_kept ? min(c * kChunk + kChunk - 1, kept - 1) : min(first(c) + kChunk - 1, pos);
+  }
 };
 
 // One chunk by itself: keys c0 .. hi of the token's request.  Leaves m_c, l_c and the thread's sums a_c.
@@ -174,8 +192,8 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
   const int kvh = h / (sh.nh / sh.nkv);
   const int pos = positions[t];
   const int32_t* table = tables + (size_t)tok_seq[t] * sh.table_stride;
-  const int lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
-  const int n_chunks = (pos - lo) / kChunk + 1;
+  const Chunks ch(sh, pos);
+  const int n_chunks = ch.n;
   const int tid = threadIdx.x;
   if (SPLIT && (int)blockIdx.y >= n_chunks) return;
 
@@ -183,9 +201,9 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
   __syncthreads();
 
   if (SPLIT) {
-    const int c = blockIdx.y, c0 = lo + c * kChunk;
+    const int c = blockIdx.y, c0 = ch.first(c);
     float m_c, l_c, a_c[PER];
-    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, min(c0 + kChunk - 1, pos), m_c, l_c, a_c);
+    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, ch.last(c, pos), m_c, l_c, a_c);
     float* cell = ws + ((size_t)blockIdx.x * max_chunks + c) * ws_stride(PER);
 #pragma unroll
     for (int u = 0; u < PER; ++u) cell[u * kChunk + tid] = a_c[u];
@@ -200,9 +218,9 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
 #pragma unroll
   for (int u = 0; u < PER; ++u) acc[u] = 0.f;
   for (int c = 0; c < n_chunks; ++c) {
-    const int c0 = lo + c * kChunk;
+    const int c0 = ch.first(c);
     float m_c, l_c, a_c[PER];
-    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, min(c0 + kChunk - 1, pos), m_c, l_c, a_c);
+    chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, ch.last(c, pos), m_c, l_c, a_c);
     merge_chunk<PER>(r, acc, m_c, l_c, a_c);
   }
   finish<T, PER>(sh, comb, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
@@ -406,17 +424,17 @@ __global__ __launch_bounds__(kChunk) void attention_plain_group_kernel(
     const int t = first + j;
     const int pos = positions[t];
     const int32_t* table = tables + (size_t)tok_seq[t] * sh.table_stride;
-    const int lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
-    const int n_chunks = (pos - lo) / kChunk + 1;
+    const Chunks ch(sh, pos);
+    const int n_chunks = ch.n;
     Running r{-INFINITY, 0.f};
     float acc[PER];
 #pragma unroll
     for (int u = 0; u < PER; ++u) acc[u] = 0.f;
     for (int c = 0; c < n_chunks; ++c) {
-      const int c0 = lo + c * kChunk;
+      const int c0 = ch.first(c);
       float m_c, l_c, a_c[PER];
       chunk_alone<T, PER>(sh, qs + j * sh.hd, es, scratch + kGroup * 4, table, k_pages, v_pages, kvh, c0,
-                          min(c0 + kChunk - 1, pos), m_c, l_c, a_c);
+                          ch.last(c, pos), m_c, l_c, a_c);
       merge_chunk<PER>(r, acc, m_c, l_c, a_c);
     }
     finish<T, PER>(sh, comb, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
@@ -432,8 +450,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_merge_kernel(T* __rest
   extern __shared__ float smem[];   // [hd * page_size / 4]
   const int t = blockIdx.x / sh.nh, h = blockIdx.x % sh.nh;
   const int pos = positions[t];
-  const int lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
-  const int n_chunks = min((pos - lo) / kChunk + 1, max_chunks);   // (never beyond what the workspace holds)
+  const int n_chunks = min(Chunks(sh, pos).n, max_chunks);   // (never beyond what the workspace holds)
   const int tid = threadIdx.x;
   Running r{-INFINITY, 0.f};
   float acc[PER];
@@ -504,11 +521,11 @@ int launch_by_pairs(int per, const void* q, int q_stride, void* out, int out_str
 
 // Floats of workspace that the chunk-by-chunk form needs for n tokens whose longest context (keys a token reads) is
 // max_context, or 0 where the sizes are refused anyway.
-extern "C" long long gb_attention_plain_split_floats(int n, int nh, int hd, int page_size, int max_context) {
+extern "C" long long gb_attention_plain_split_floats(int n, int nh, int hd, int page_size, int max_context, int keep_first) {
   if (n <= 0 || nh <= 0 || hd <= 0 || page_size <= 0 || page_size % 4 || max_context <= 0) return 0;
   const int per = own_pairs(hd, page_size);
   if (per == 0) return 0;
-  const long long chunks = (max_context + kChunk - 1) / kChunk;
+  const long long chunks = (max_context + kChunk - 1) / kChunk + (keep_first > 0 ? 1 : 0);
   return (long long)n * nh * chunks * (per * kChunk + 2);
 }
 
@@ -520,13 +537,14 @@ extern "C" long long gb_attention_plain_split_floats(int n, int nh, int hd, int 
 extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int out_stride, int dtype,
                                   const int32_t* positions, const int32_t* tok_seq, const int32_t* tables,
                                   int table_stride, const void* k_pages, const void* v_pages, int n, int nh, int nkv,
-                                  int hd, int page_size, float scale, int window, float* ws, long long ws_floats,
-                                  int max_context, int grouped, hipStream_t stream) {
+                                  int hd, int page_size, float scale, int window, int keep_first, float* ws,
+                                  long long ws_floats, int max_context, int grouped, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_plain: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh, nkv, hd);
   GB_REQUIRE(nh % nkv == 0, "attention_plain: %d query heads are not a multiple of %d key heads", nh, nkv);
   GB_REQUIRE(hd <= kChunk, "attention_plain: head size %d is above the supported 256", hd);
   GB_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd, "attention_plain: row strides shorter than the heads");
   GB_REQUIRE(page_size > 0 && table_stride > 0 && window >= 0, "attention_plain: bad page size, table stride or window");
+  GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_plain: kept first keys go with a window");
   GB_REQUIRE(page_size % 4 == 0, "attention_plain: a page of %d tokens is not whole words of four slots", page_size);
   GB_REQUIRE((long long)n * nh < (1ll << 31), "attention_plain: too many (token, head) pairs");
   const int per = own_pairs(hd, page_size);
@@ -536,13 +554,14 @@ extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int ou
   int max_chunks = 0;
   if (ws != nullptr) {
     GB_REQUIRE(max_context > 0, "attention_plain: the chunk-by-chunk form needs the longest context");
-    max_chunks = (max_context + kChunk - 1) / kChunk;
+    // (a token's chunks of kept first keys and of its window are whole chunks each: one more than its keys may fill)
+    max_chunks = (max_context + kChunk - 1) / kChunk + (keep_first > 0 ? 1 : 0);
     GB_REQUIRE(max_chunks <= 65535, "attention_plain: a context of %d keys is more chunks than a launch takes", max_context);
-    GB_REQUIRE(ws_floats >= gb_attention_plain_split_floats(n, nh, hd, page_size, max_context),
+    GB_REQUIRE(ws_floats >= gb_attention_plain_split_floats(n, nh, hd, page_size, max_context, keep_first),
                "attention_plain: the workspace holds %lld floats, %lld are needed", ws_floats,
-               gb_attention_plain_split_floats(n, nh, hd, page_size, max_context));
+               gb_attention_plain_split_floats(n, nh, hd, page_size, max_context, keep_first));
   }
-  const Shape sh{nh, nkv, hd, page_size, window, table_stride, scale};
+  const Shape sh{nh, nkv, hd, page_size, window, table_stride, scale, keep_first};
   if (dtype == kF32)
     return launch_by_pairs<float>(per, q, q_stride, out, out_stride, positions, tok_seq, tables, k_pages, v_pages, n, sh, ws,
                                   max_chunks, grouped != 0, stream);

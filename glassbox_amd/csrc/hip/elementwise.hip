@@ -10,27 +10,32 @@ using namespace gb;
 GB_DEFINE_LAST_ERROR
 
 // ---------------------------------------------------------------- embedding gather
-// x[i, :] = table[ids[i], :]   (crates/glassbox-core/src/model.rs:228-231)
+// x[c, i, :] = table[ids[i], :] * scale for each of `copies` copies   (crates/glassbox-core/src/model.rs:228-231;
+// a scale of 1 and one copy there)
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids, float* __restrict__ x,
-                             int d, int vocab) {
+                             int n, int d, int vocab, float scale, int copies) {
   const int i = blockIdx.x;
   int id = ids[i];
   const bool ok = id >= 0 && id < vocab;
   const T* row = table + (size_t)(ok ? id : 0) * d;
-  for (int c = threadIdx.x; c < d; c += blockDim.x)
-    x[(size_t)i * d + c] = ok ? to_f(row[c]) : __builtin_nanf("");  // a bad id must not pass silently
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    const float v = ok ? to_f(row[c]) * scale : __builtin_nanf("");  // a bad id must not pass silently
+    for (int k = 0; k < copies; ++k) x[((size_t)k * n + i) * d + c] = v;
+  }
 }
 
 extern "C" int gb_embed(const void* table, int table_dtype, const int32_t* ids, float* x, int n, int d, int vocab,
-                        hipStream_t stream) {
-  GB_REQUIRE(n >= 0 && d > 0 && vocab > 0, "embed: bad sizes n=%d d=%d vocab=%d", n, d, vocab);
+                        float scale, int copies, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && d > 0 && vocab > 0 && copies > 0, "embed: bad sizes n=%d d=%d vocab=%d copies=%d", n, d, vocab, copies);
   if (n == 0) return 0;
   const int threads = d >= 256 ? 256 : 64;
   if (table_dtype == kF32)
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)table, ids, x, d, vocab);
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)table, ids, x, n, d, vocab,
+                       scale, copies);
   else if (table_dtype == kBF16)
-    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)table, ids, x, d, vocab);
+    hipLaunchKernelGGL(embed_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)table, ids, x, n, d, vocab,
+                       scale, copies);
   else
     return fail("embed: unknown table dtype %d", table_dtype);
   return launched("embed");
@@ -590,6 +595,112 @@ extern "C" int gb_copy_rows(void* base, long long row_bytes, const int32_t* src,
   return launched("copy_rows");
 }
 
+
+// ------------------------------------------------------------- query/key norm and cache write
+// For attention whose values are its keys as projected: row t of `qk` holds nh query heads, then nkv key heads.
+// x = projection + bias; a key head's x goes to the value pages as it is; then every head is RMS-normed over its
+// hd dimensions with a weight shared by the heads (w_q for queries, w_k for keys): queries are written back in
+// place, keys into the key pages.  One wave a (token, head); sums and the norm in 32-bit.
+template <typename T>
+__global__ __launch_bounds__(kWave) void qk_norm_store_kernel(T* __restrict__ qk, int stride, const float* __restrict__ bias_q,
+                                                            const float* __restrict__ bias_k, const float* __restrict__ w_q,
+                                                            const float* __restrict__ w_k, float eps,
+                                                            const int32_t* __restrict__ slots, T* __restrict__ k_pages,
+                                                            T* __restrict__ v_pages, int nh, int nkv, int hd, int page_size) {
+  const int t = blockIdx.x / (nh + nkv), h = blockIdx.x % (nh + nkv);
+  const bool is_key = h >= nh;
+  const int lane = threadIdx.x;
+  T* row = qk + (size_t)t * stride + (size_t)h * hd;
+  const float* bias = is_key ? (bias_k ? bias_k + (size_t)(h - nh) * hd : nullptr) : (bias_q ? bias_q + (size_t)h * hd : nullptr);
+  const float* w = is_key ? w_k : w_q;
+  constexpr int kMax = 4;   // head sizes up to 256
+  float x[kMax];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < kMax; ++j) {
+    const int d = lane + j * kWave;
+    x[j] = 0.f;
+    if (d < hd) {
+      x[j] = to_f(row[d]) + (bias ? bias[d] : 0.f);
+      // what the projection gives in this type, bias included, is the value and the norm's operand alike
+      x[j] = to_f(from_f<T>(x[j]));
+      ss = fmaf(x[j], x[j], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float s = w ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.0f;
+  const int slot = is_key && slots ? slots[t] : -1;
+  const int piece = key_piece(hd);
+  T* kb = nullptr;
+  T* vb = nullptr;
+  if (slot >= 0) {
+    const size_t block = ((size_t)(slot / page_size) * nkv + (h - nh)) * (size_t)page_size * hd;
+    kb = k_pages + block;
+    vb = v_pages + block;
+  }
+#pragma unroll
+  for (int j = 0; j < kMax; ++j) {
+    const int d = lane + j * kWave;
+    if (d >= hd) continue;
+    const float y = w ? w[d] * (x[j] * s) : x[j];
+    if (!is_key) {
+      row[d] = from_f<T>(y);
+    } else if (slot >= 0) {
+      kb[key_offset(slot % page_size, d, page_size, piece)] = from_f<T>(y);
+      vb[(size_t)d * page_size + slot % page_size] = from_f<T>(x[j]);
+    }
+  }
+}
+
+extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bias_q, const float* bias_k, const float* w_q,
+                                const float* w_k, float eps, const int32_t* slots, void* k_pages, void* v_pages, int n,
+                                int nh, int nkv, int hd, int page_size, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && hd > 0 && hd <= 4 * kWave, "qk_norm_store: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh,
+             nkv, hd);
+  GB_REQUIRE(stride >= (nh + nkv) * hd, "qk_norm_store: rows of %d hold fewer than %d heads of %d", stride, nh + nkv, hd);
+  GB_REQUIRE(slots == nullptr || (k_pages && v_pages && page_size > 0), "qk_norm_store: cache rows without pages");
+  GB_REQUIRE((long long)n * (nh + nkv) < (1ll << 31), "qk_norm_store: too many (token, head) pairs");
+  if (n == 0) return 0;
+  const dim3 grid((unsigned)(n * (nh + nkv)));
+  if (dtype == kF32)
+    hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, dim3(kWave), 0, stream, (float*)qk, stride, bias_q, bias_k, w_q, w_k,
+                       eps, slots, (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, dim3(kWave), 0, stream, (bf16*)qk, stride, bias_q, bias_k, w_q, w_k, eps,
+                       slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size);
+  else
+    return fail("qk_norm_store: unknown dtype %d", dtype);
+  return launched("qk_norm_store");
+}
+
+// ------------------------------------------------------------------------ scale
+// x *= s   (float32: logits that a model scales)
+__global__ void scale_rows_kernel(float* __restrict__ x, float s, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) x[i] *= s;
+}
+
+extern "C" int gb_scale_rows(float* x, float s, long long count, hipStream_t stream) {
+  GB_REQUIRE(count >= 0 && (count + 255) / 256 < (1ll << 31), "scale_rows: bad size %lld", count);
+  if (count == 0) return 0;
+  hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, x, s, count);
+  return launched("scale_rows");
+}
+
+// ------------------------------------------------------------------------ bias
+// x[r, :] += bias   (float32 rows: the output of a projection that has a bias)
+__global__ void add_bias_kernel(float* __restrict__ x, const float* __restrict__ bias, int d) {
+  float* row = x + (size_t)blockIdx.x * d;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) row[c] += bias[c];
+}
+
+extern "C" int gb_add_bias(float* x, const float* bias, int n, int d, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && d > 0, "add_bias: bad sizes n=%d d=%d", n, d);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(add_bias_kernel, dim3(n), dim3(d >= 256 ? 256 : 64), 0, stream, x, bias, d);
+  return launched("add_bias");
+}
+
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_embed)
 GB_TAPED(gb_rmsnorm)
@@ -597,3 +708,6 @@ GB_TAPED(gb_rope_table)
 GB_TAPED(gb_rope_store)
 GB_TAPED(gb_silu_mul)
 GB_TAPED(gb_copy_rows)
+GB_TAPED(gb_qk_norm_store)
+GB_TAPED(gb_add_bias)
+GB_TAPED(gb_scale_rows)

@@ -1,0 +1,296 @@
+// Linear attention with a decayed matrix state per (request, head): retention (one fixed decay a head) and
+// gated linear attention (a decay per key channel and token).
+//
+//   S_t = diag(a_t) S_(t-1) + k_t v_t^T      S: [dk, dv], a_t: one number a head, or a vector over the dk rows
+//   o_t = S_t^T q_t
+//
+// The state is 32-bit and lives in a slot per live request, [heads, dv, dk]: a column of S (one value channel)
+// lies in a row of memory.  Columns never meet: column j of S_t depends on column j of S_(t-1), k_t and v_t[j]
+// alone.  So a wave owns eight columns, eight lanes a column, a lane R = ceil(dk / 8) of its rows in registers, and
+// walks its request's tokens of the step in order: the same additions in the same order whether a prompt comes
+// whole, in portions or token by token.  A workgroup (four waves, 32 columns of one head) stages the tokens'
+// q, k and decays through LDS sixteen tokens at a time, the next sixteen on their way from memory meanwhile.
+// q, k and the decays come in 32-bit (what the kernels below prepare), v in the activations' type.
+//
+// Around it: `retention_prep` (rotation of the first `rot` dimensions of the q and k heads in rotate-half pairs,
+// k scaled), `gla_prep` (q scaled, decays sigmoid(z)^(1/tau) from the low-rank projection z = A2 t + b), and
+// `head_norm_gate` (each head's output divided by its root mean square, an optional weight over dv, times
+// silu(gate), written in the activations' type for the output projection).
+#include "common.h"
+
+using namespace gb;
+
+GB_DEFINE_LAST_ERROR
+
+namespace {
+
+constexpr int kTokens = 16;    // tokens staged at a time
+constexpr int kLanesCol = 8;   // lanes a column of the state
+constexpr int kColsWave = kWave / kLanesCol;
+constexpr int kWaves = 4;
+constexpr int kColsBlock = kColsWave * kWaves;
+constexpr int kThreads = kWaves * kWave;
+
+template <typename T, int R, bool GATED>
+__global__ __launch_bounds__(kThreads) void scan_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ a, const float* __restrict__ head_decay,
+    const T* __restrict__ v, int v_stride, float* __restrict__ out, float* __restrict__ state,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slots, int nh, int dk, int dv) {
+  constexpr int DKP = R * kLanesCol;                       // rows, padded
+  constexpr int PER = (kTokens * DKP) / kThreads;          // staged elements a thread and array (R >= 2)
+  __shared__ float qs[kTokens][DKP], ks[kTokens][DKP], ds[GATED ? kTokens : 1][GATED ? DKP : 1];
+  __shared__ float vs[kTokens][kColsBlock];
+  const int seq = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kColsBlock;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int rg = lane % kLanesCol;                          // which R rows of the column
+  const int cb = wave * kColsWave + lane / kLanesCol;       // column within the block
+  const int col = col0 + cb;
+  const int first = q_start[seq], count = q_len[seq];
+  const int width = nh * dk;
+  const bool live = col < dv;
+
+  float S[R];
+  float* srow = state + (((size_t)state_slots[seq] * nh + h) * dv + (live ? col : 0)) * dk + rg * R;
+  const bool fresh = pos0[seq] == 0;   // a request's first tokens start from an empty state, whatever the slot held
+#pragma unroll
+  for (int m = 0; m < R; ++m) S[m] = (!fresh && live && rg * R + m < dk) ? srow[m] : 0.f;
+  const float decay = GATED ? 1.f : head_decay[h];
+
+  float nq[PER], nk[PER], na[GATED ? PER : 1], nv[2];
+  auto fetch = [&](int t0) {   // tokens t0 .. t0 + kTokens - 1 of this request's rows into registers
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int idx = tid + e * kThreads, tok = idx / DKP, ch = idx % DKP;
+      const bool ok = t0 + tok < count && ch < dk;
+      const size_t at = (size_t)(first + t0 + tok) * width + (size_t)h * dk + ch;
+      nq[e] = ok ? q[at] : 0.f;
+      nk[e] = ok ? k[at] : 0.f;
+      if (GATED) na[e] = ok ? a[at] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int idx = tid + e * kThreads, tok = idx / kColsBlock, c = idx % kColsBlock;
+      const bool ok = t0 + tok < count && col0 + c < dv;
+      nv[e] = ok ? to_f(v[(size_t)(first + t0 + tok) * v_stride + (size_t)h * dv + col0 + c]) : 0.f;
+    }
+  };
+  static_assert(kTokens * kColsBlock == 2 * kThreads, "two staged values of v a thread");
+
+  fetch(0);
+  for (int t0 = 0; t0 < count; t0 += kTokens) {
+    __syncthreads();   // the tokens before have been read
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int idx = tid + e * kThreads;
+      (&qs[0][0])[idx] = nq[e];
+      (&ks[0][0])[idx] = nk[e];
+      if (GATED) (&ds[0][0])[idx] = na[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 2; ++e) (&vs[0][0])[tid + e * kThreads] = nv[e];
+    __syncthreads();
+    if (t0 + kTokens < count) fetch(t0 + kTokens);
+    const int here = min(kTokens, count - t0);
+    for (int j = 0; j < here; ++j) {
+      const float vv = vs[j][cb];
+      float part = 0.f;
+#pragma unroll
+      for (int m = 0; m < R; ++m) {
+        const float kk = ks[j][rg * R + m], qq = qs[j][rg * R + m];
+        const float aa = GATED ? ds[j][rg * R + m] : decay;
+        S[m] = fmaf(aa, S[m], kk * vv);
+        part = fmaf(S[m], qq, part);
+      }
+      // the eight lanes of a column, in a fixed order
+      part += __shfl_xor(part, 1, kWave);
+      part += __shfl_xor(part, 2, kWave);
+      part += __shfl_xor(part, 4, kWave);
+      if (rg == 0 && live) out[(size_t)(first + t0 + j) * ((size_t)nh * dv) + (size_t)h * dv + col] = part;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int m = 0; m < R; ++m)
+      if (rg * R + m < dk) srow[m] = S[m];
+  }
+}
+
+// q32, k32 [n, nh * dk] from the q and k heads of the projection's rows: dimensions i < rot of a head in pairs
+// (i, i + rot / 2), i < rot / 2, turned by the row's angles (cos, sin [n, rot / 2]); the rest as they are; k times k_scale.
+template <typename T>
+__global__ void retention_prep_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off,
+                                      const float* __restrict__ cosv, const float* __restrict__ sinv, float* __restrict__ q32,
+                                      float* __restrict__ k32, int nh, int dk, int rot, float k_scale) {
+  const int t = blockIdx.x, width = nh * dk, half = rot / 2;
+  const T* row = proj + (size_t)t * stride;
+  for (int e = threadIdx.x; e < 2 * width; e += blockDim.x) {
+    const bool is_k = e >= width;
+    const int c = is_k ? e - width : e, d = c % dk;
+    const T* src = row + (is_k ? k_off : q_off);
+    float x = to_f(src[c]);
+    if (d < rot) {
+      const bool lower = d < half;
+      const int i = lower ? d : d - half;
+      const float other = to_f(src[lower ? c + half : c - half]);
+      const float cs = cosv[(size_t)t * half + i], sn = sinv[(size_t)t * half + i];
+      // (u, w) -> (u cos - w sin, w cos + u sin)
+      x = lower ? x * cs - other * sn : x * cs + other * sn;
+    }
+    if (is_k) k32[(size_t)t * width + c] = x * k_scale;
+    else q32[(size_t)t * width + c] = x;
+  }
+}
+
+__device__ __forceinline__ float log_sigmoid(float z) {
+  // log(1 / (1 + exp(-z))) without overflow on either side
+  return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+}
+
+// q32 = q * q_scale, k32 = k, decay[t, c] = sigmoid(z)^(1/tau) with z = sum_r A2[c, r] low[t, r] + b[c]
+template <typename T>
+__global__ void gla_prep_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int low_off,
+                                const T* __restrict__ a2, const float* __restrict__ a2_bias, float* __restrict__ q32,
+                                float* __restrict__ k32, float* __restrict__ decay, int width, int rank, float q_scale,
+                                float inv_tau) {
+  extern __shared__ float low[];   // [rank]
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * stride;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = to_f(row[low_off + r]);
+  __syncthreads();
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    q32[(size_t)t * width + c] = to_f(row[q_off + c]) * q_scale;
+    k32[(size_t)t * width + c] = to_f(row[k_off + c]);
+    float z = 0.f;
+    const T* w = a2 + (size_t)c * rank;
+    for (int r = 0; r < rank; ++r) z = fmaf(to_f(w[r]), low[r], z);
+    z += a2_bias ? a2_bias[c] : 0.f;
+    decay[(size_t)t * width + c] = expf(log_sigmoid(z) * inv_tau);
+  }
+}
+
+// out[t, h, :] = w * o / sqrt(mean(o^2) + eps) * silu(gate[t, h, :])  (w == nullptr: no weight).  One wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                             int gate_stride, const float* __restrict__ w,
+                                                             T* __restrict__ out, int nh, int dv, float eps) {
+  const int t = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
+  const float* orow = o + ((size_t)t * nh + h) * dv;
+  float ss = 0.f;
+  for (int d = lane; d < dv; d += kWave) ss = fmaf(orow[d], orow[d], ss);
+  ss = wave_sum(ss);
+  const float s = 1.0f / sqrtf(ss / (float)dv + eps);
+  for (int d = lane; d < dv; d += kWave) {
+    const float g = to_f(gate[(size_t)t * gate_stride + (size_t)h * dv + d]);
+    const float act = g / (1.0f + expf(-g));
+    const float y = (w ? w[d] : 1.0f) * (orow[d] * s);
+    out[((size_t)t * nh + h) * dv + d] = from_f<T>(y * act);
+  }
+}
+
+template <typename T, bool GATED>
+int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const float* k, const float* a, const float* head_decay,
+                const void* v, int v_stride, float* out, float* state, const int32_t* q_start, const int32_t* q_len,
+                const int32_t* pos0, const int32_t* slots, int nh, int dk, int dv) {
+#define GB_SCAN(RR)                                                                                                          \
+  case RR:                                                                                                                   \
+    hipLaunchKernelGGL((scan_kernel<T, RR, GATED>), grid, dim3(kThreads), 0, stream, q, k, a, head_decay, (const T*)v, v_stride, \
+                       out, state, q_start, q_len, pos0, slots, nh, dk, dv);                                                 \
+    break;
+  switch (R) {
+    GB_SCAN(2) GB_SCAN(4) GB_SCAN(8) GB_SCAN(16) GB_SCAN(32)
+    default: return fail("linear_scan: no kernel for %d rows a lane", R);
+  }
+#undef GB_SCAN
+  return launched("linear_scan");
+}
+
+}  // namespace
+
+// The recurrence over the rows of a step.  q, k [n, nh * dk] float32; `a` [n, nh * dk] float32 decays a key channel, or
+// nullptr with head_decay [nh] float32; v rows of nh * dv in the activations' type (row stride v_stride); out [n, nh * dv]
+// float32; state [slots, nh, dv, dk] float32.  Request s of the step brings rows q_start[s] .. + q_len[s] - 1, starts at
+// position pos0[s] (0: from an empty state) and keeps its state in slot state_slots[s].
+extern "C" int gb_linear_scan(const float* q, const float* k, const float* a, const float* head_decay, const void* v,
+                              int v_dtype, int v_stride, float* out, float* state, const int32_t* q_start,
+                              const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
+                              int dk, int dv, hipStream_t stream) {
+  GB_REQUIRE(n_seqs >= 0 && nh > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes requests=%d heads=%d dk=%d dv=%d", n_seqs, nh, dk, dv);
+  GB_REQUIRE(dk <= 32 * kLanesCol, "linear_scan: a key size of %d is above the supported %d", dk, 32 * kLanesCol);
+  GB_REQUIRE((a != nullptr) != (head_decay != nullptr), "linear_scan: a decay a head or a decay a key channel, one of the two");
+  GB_REQUIRE(v_stride >= nh * dv, "linear_scan: value rows of %d hold fewer than %d heads of %d", v_stride, nh, dv);
+  GB_REQUIRE(n_seqs <= 65535 && nh <= 65535, "linear_scan: too many requests or heads for one launch");
+  if (n_seqs == 0) return 0;
+  int R = 2;
+  while (R * kLanesCol < dk) R *= 2;
+  const dim3 grid((unsigned)((dv + kColsBlock - 1) / kColsBlock), (unsigned)nh, (unsigned)n_seqs);
+  const bool gated = a != nullptr;
+  if (v_dtype == kF32)
+    return gated ? launch_scan<float, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv)
+                 : launch_scan<float, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv);
+  if (v_dtype == kBF16)
+    return gated ? launch_scan<bf16, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv)
+                 : launch_scan<bf16, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv);
+  return fail("linear_scan: unknown dtype %d", v_dtype);
+}
+
+extern "C" int gb_retention_prep(const void* proj, int dtype, int stride, int q_off, int k_off, const float* cosv,
+                                 const float* sinv, float* q32, float* k32, int n, int nh, int dk, int rot, float k_scale,
+                                 hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh > 0 && dk > 0 && rot >= 0 && rot <= dk && rot % 2 == 0, "retention_prep: bad sizes n=%d heads=%d dk=%d rot=%d",
+             n, nh, dk, rot);
+  GB_REQUIRE(q_off >= 0 && k_off >= 0 && q_off + nh * dk <= stride && k_off + nh * dk <= stride, "retention_prep: heads beyond the row");
+  GB_REQUIRE(rot == 0 || (cosv && sinv), "retention_prep: rotation without tables");
+  if (n == 0) return 0;
+  const int threads = nh * dk >= 512 ? 256 : 128;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(retention_prep_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)proj, stride, q_off, k_off,
+                       cosv, sinv, q32, k32, nh, dk, rot, k_scale);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(retention_prep_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)proj, stride, q_off, k_off,
+                       cosv, sinv, q32, k32, nh, dk, rot, k_scale);
+  else
+    return fail("retention_prep: unknown dtype %d", dtype);
+  return launched("retention_prep");
+}
+
+extern "C" int gb_gla_prep(const void* proj, int dtype, int stride, int q_off, int k_off, int low_off, const void* a2,
+                           const float* a2_bias, float* q32, float* k32, float* decay, int n, int width, int rank,
+                           float q_scale, float inv_tau, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && width > 0 && rank > 0 && rank <= 4096, "gla_prep: bad sizes n=%d width=%d rank=%d", n, width, rank);
+  GB_REQUIRE(q_off >= 0 && k_off >= 0 && low_off >= 0 && q_off + width <= stride && k_off + width <= stride &&
+                 low_off + rank <= stride, "gla_prep: heads beyond the row");
+  if (n == 0) return 0;
+  const int threads = width >= 512 ? 256 : 128;
+  const size_t smem = sizeof(float) * rank;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(gla_prep_kernel<float>, dim3(n), dim3(threads), smem, stream, (const float*)proj, stride, q_off, k_off,
+                       low_off, (const float*)a2, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(gla_prep_kernel<bf16>, dim3(n), dim3(threads), smem, stream, (const bf16*)proj, stride, q_off, k_off,
+                       low_off, (const bf16*)a2, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
+  else
+    return fail("gla_prep: unknown dtype %d", dtype);
+  return launched("gla_prep");
+}
+
+extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, int gate_stride, const float* w, void* out, int n,
+                                 int nh, int dv, float eps, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh > 0 && dv > 0 && gate_stride >= nh * dv, "head_norm_gate: bad sizes n=%d heads=%d dv=%d", n, nh, dv);
+  GB_REQUIRE((long long)n * nh < (1ll << 31), "head_norm_gate: too many (token, head) pairs");
+  if (n == 0) return 0;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3((unsigned)(n * nh)), dim3(kWave), 0, stream, o, (const float*)gate,
+                       gate_stride, w, (float*)out, nh, dv, eps);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16>, dim3((unsigned)(n * nh)), dim3(kWave), 0, stream, o, (const bf16*)gate,
+                       gate_stride, w, (bf16*)out, nh, dv, eps);
+  else
+    return fail("head_norm_gate: unknown dtype %d", dtype);
+  return launched("head_norm_gate");
+}
+
+GB_TAPED(gb_linear_scan)
+GB_TAPED(gb_retention_prep)
+GB_TAPED(gb_gla_prep)
+GB_TAPED(gb_head_norm_gate)

@@ -14,12 +14,13 @@ using gb::CacheManager;
 extern "C" {
 
 // ---- cache manager -------------------------------------------------------
-void* gbh_cache_create(int page_size, int n_groups, const int* kinds, const int* windows,
+void* gbh_cache_create(int page_size, int n_groups, const int* kinds, const int* windows, const int* keep_firsts,
                        const int* num_pages, int num_state_slots, int share_prefixes) {
   std::vector<gb::GroupSpec> groups(n_groups);
   for (int i = 0; i < n_groups; ++i) {
     groups[i].kind = kinds[i];
     groups[i].window = windows[i];
+    groups[i].keep_first = keep_firsts ? keep_firsts[i] : 0;
     groups[i].num_pages = num_pages[i];
   }
   return new CacheManager(page_size, groups, num_state_slots, share_prefixes != 0);

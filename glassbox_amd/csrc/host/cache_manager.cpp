@@ -192,8 +192,9 @@ int CacheManager::commit(int64_t id, const int32_t* tokens, int n) {
     int first_needed = s.len - g.spec.window + 1;  // oldest key the next query reads
     if (first_needed <= 0) continue;
     int dead = first_needed / page_size_;          // pages [0, dead) lie wholly before it
+    int kept = (g.spec.keep_first + page_size_ - 1) / page_size_;   // pages that hold a key every query reads
     auto& table = s.tables[gi];
-    for (int j = 0; j < dead && j < (int)table.size(); ++j) {
+    for (int j = kept; j < dead && j < (int)table.size(); ++j) {
       if (table[j] >= 0) {
         release(g, table[j]);
         table[j] = -1;

@@ -7,7 +7,8 @@
 // through a hash chain over full pages, copy-on-write of a shared partial page,
 // and a "cached" list of unreferenced pages that still carry a prefix hash.
 // Added here: several page groups (layers whose mixers need all keys, or only a
-// window of them, each with a pool of its own) and fixed-size state slots.
+// window of them, with or without the first few kept for good, each with a pool of its own) and fixed-size
+// state slots.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -21,6 +22,7 @@ enum GroupKind : int { kFull = 0, kWindow = 1 };
 struct GroupSpec {
   int kind = kFull;
   int window = 0;      // kWindow: a query at position p reads keys p-window+1 .. p
+  int keep_first = 0;  // kWindow: and keys 0 .. keep_first-1, whose pages are never given back while the request lives
   int num_pages = 0;
 };
 

@@ -110,13 +110,13 @@ class Engine:
         # page groups: cache layers whose mixers keep the same span of positions share page numbers
         specs = model.cache_specs()
         states = model.state_specs()
-        keys: List[Tuple[int, int]] = []
+        keys: List[Tuple[int, int, int]] = []
         for spec in specs:
             if spec is not None and spec.group_key not in keys:
                 keys.append(spec.group_key)
         self.group_keys = keys
         self.has_state = any(s is not None for s in states)
-        groups = [GroupSpec(kind, window, num_pages) for kind, window in keys]
+        groups = [GroupSpec(kind, window, num_pages, keep_first) for kind, window, keep_first in keys]
         if prefix_caching:
             obstacles = sharing_obstacles(model)
             if obstacles:

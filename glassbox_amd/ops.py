@@ -40,7 +40,7 @@ def dtype_code(t: torch.Tensor) -> int:
 
 _SIGS = {
     "elementwise": {
-        "gb_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
+        "gb_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp],
         "gb_rmsnorm": [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
         "gb_rope_table": [_vp, _vp, _vp, _vp, _i, _i, _vp],
         # qkv, dtype, stride, cos, sin, slots, k, v, n, nh, nkv, hd, page, rotate, v_rows, q_start, q_len, pos0,
@@ -48,6 +48,26 @@ _SIGS = {
         "gb_rope_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp],
         "gb_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
         "gb_copy_rows": [_vp, C.c_longlong, _vp, _vp, _i, _vp],
+        # qk, dtype, stride, bias_q, bias_k, w_q, w_k, eps, slots, k, v, n, nh, nkv, hd, page, stream
+        "gb_qk_norm_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+        "gb_add_bias": [_vp, _vp, _i, _i, _vp],
+        "gb_scale_rows": [_vp, _f, C.c_longlong, _vp],
+    },
+    "streams": {
+        # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, stream
+        "gb_streams_norm": [_vp, C.c_longlong, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _f, _vp],
+        "gb_streams_mix": [_vp, C.c_longlong, _i, _vp, _vp, _vp, C.c_longlong, _vp],
+    },
+    "linear_attention": {
+        # q, k, decays, head decays, v, v dtype, v stride, out, state, q_start, q_len, pos0, state slots, requests, heads,
+        # dk, dv, stream
+        "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+        # proj, dtype, stride, q_off, k_off, cos, sin, q32, k32, n, heads, dk, rot, k_scale, stream
+        "gb_retention_prep": [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
+        # proj, dtype, stride, q_off, k_off, low_off, a2, a2 bias, q32, k32, decay, n, width, rank, q_scale, 1/tau, stream
+        "gb_gla_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _vp],
+        # o, gate, dtype, gate stride, w, out, n, heads, dv, eps, stream
+        "gb_head_norm_gate": [_vp, _vp, _i, _i, _vp, _vp, _i, _i, _i, _f, _vp],
     },
     "gemm_f32": {
         "gb_gemm_f32": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
@@ -69,9 +89,10 @@ _SIGS = {
     "attention_plain": {
         # q, q_stride, out, out_stride, dtype, positions, tok_seq, tables, table_stride, k, v, n, nh, nkv, hd, page,
         # scale, window, workspace, workspace floats, max_context, stream
-        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp,
+        # scale, window, kept first keys, workspace, workspace floats, max_context, grouped, stream
+        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp,
                                C.c_longlong, _i, _i, _vp],
-        "gb_attention_plain_split_floats": [_i, _i, _i, _i, _i],
+        "gb_attention_plain_split_floats": [_i, _i, _i, _i, _i, _i],
     },
     "attention_bf16": {
         # q, q_stride, out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k, v,
@@ -335,15 +356,17 @@ def _check_pages(k_pages, v_pages, dtype, what: str):
 
 
 # ------------------------------------------------------------------ elementwise
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[i, :] = table[ids[i], :] as 32-bit floats."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[i, :] = table[ids[i], :] * scale as 32-bit floats; an out of [copies, n, d] receives that many copies."""
     _dev(table, ids, out)
-    n, d = out.shape
+    copies = out.shape[0] if out.dim() == 3 else 1
+    n, d = out.shape[-2:]
     _i32(ids, "ids", n)
     if out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous() or table.shape[1] != d:
-        raise KernelError("embed: out must be contiguous float32 [n, d] and table [vocab, d]")
+        raise KernelError("embed: out must be contiguous float32 [n, d] or [copies, n, d] and table [vocab, d]")
     lib = _lib("elementwise")
-    _launch(lib, lib.gb_embed, _p(table), dtype_code(table), _p(ids), _p(out), n, d, table.shape[0], _stream())
+    _launch(lib, lib.gb_embed, _p(table), dtype_code(table), _p(ids), _p(out), n, d, table.shape[0], float(scale),
+            int(copies), _stream())
 
 
 def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float, out: torch.Tensor,
@@ -437,6 +460,198 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
     row_bytes = base[0].numel() * base.element_size()
     lib = _lib("elementwise")
     _launch(lib, lib.gb_copy_rows, _p(base), row_bytes, _p(src), _p(dst), count, _stream())
+
+
+def qk_norm_store(qk: torch.Tensor, bias_q: Optional[torch.Tensor], bias_k: Optional[torch.Tensor],
+                  w_q: Optional[torch.Tensor], w_k: Optional[torch.Tensor], eps: float, slots: Optional[torch.Tensor],
+                  k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv_heads: int,
+                  head_dim: int) -> None:
+    """Rows of query heads then key heads: adds the biases, writes each key head as it then is to the value pages
+    (the values of such a layer are its keys as projected), RMS-norms every head over its dimensions with the weight
+    that the heads of its kind share (None: the head stays as it is), and leaves queries in place and keys in the key
+    pages at ``slots`` (None: nothing is stored).  Biases and weights are float32."""
+    _dev(qk, bias_q, bias_k, w_q, w_k, slots, k_pages, v_pages)
+    n = qk.shape[0]
+    stride = _rows(qk, "qk")
+    for t, size, what in ((bias_q, n_heads * head_dim, "bias_q"), (bias_k, n_kv_heads * head_dim, "bias_k"),
+                          (w_q, head_dim, "w_q"), (w_k, head_dim, "w_k")):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != size):
+            raise KernelError(f"qk_norm_store: {what} must be contiguous float32 of {size} entries")
+    if qk.shape[1] < (n_heads + n_kv_heads) * head_dim:
+        raise KernelError("qk_norm_store: rows shorter than the heads")
+    page_size = 0
+    if slots is not None:
+        _i32(slots, "slots", n)
+        _, p_heads, page_size, p_hd = _check_pages(k_pages, v_pages, qk.dtype, "qk_norm_store")
+        if (p_heads, p_hd) != (n_kv_heads, head_dim):
+            raise KernelError("qk_norm_store: pages do not have this layer's kv heads and head size")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_qk_norm_store, _p(qk), dtype_code(qk), stride, _p(bias_q), _p(bias_k), _p(w_q), _p(w_k), float(eps),
+            _p(slots), _p(k_pages), _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size, _stream())
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """x[r, :] += bias, both float32."""
+    _dev(x, bias)
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or bias.dtype != torch.float32 or bias.numel() != d \
+            or not bias.is_contiguous():
+        raise KernelError("add_bias: x must be contiguous float32 [n, d] and bias float32 [d]")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_add_bias, _p(x), _p(bias), n, d, _stream())
+
+
+def scale_rows(x: torch.Tensor, s: float) -> None:
+    """x *= s, float32."""
+    _dev(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("scale_rows: x must be contiguous float32")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_scale_rows, _p(x), float(s), x.numel(), _stream())
+
+
+# ------------------------------------------------------------------- residual streams
+MAX_STREAMS = 8   # streams.hip keeps a row's streams in registers
+
+
+def _streams(X: torch.Tensor, what: str):
+    if X.dim() != 3 or X.dtype != torch.float32 or not X.is_contiguous() or not 1 <= X.shape[0] <= MAX_STREAMS:
+        raise KernelError(f"{what}: the streams must be contiguous float32 [streams <= {MAX_STREAMS}, n, d]")
+    return X.shape
+
+
+def streams_norm(X: torch.Tensor, w_in: Optional[torch.Tensor], gamma: torch.Tensor, eps: float, out: torch.Tensor,
+                 rows: Optional[torch.Tensor] = None, total: Optional[torch.Tensor] = None) -> None:
+    """out[r] = gamma * u / sqrt(mean(u^2) + eps), u = sum_s w_in[s] X[s][rows[r] or r] (``w_in`` None: the plain sum of
+    the streams); ``total`` (float32 [m, d]) receives u as well."""
+    _dev(X, w_in, gamma, out, rows, total)
+    S, n, d = _streams(X, "streams_norm")
+    m = out.shape[0]
+    if out.shape != (m, d) or not out.is_contiguous() or gamma.numel() != d or not gamma.is_contiguous():
+        raise KernelError("streams_norm: out must be contiguous [m, d] and gamma hold d entries")
+    if w_in is not None and (w_in.dtype != torch.float32 or w_in.numel() != S or not w_in.is_contiguous()):
+        raise KernelError("streams_norm: w_in must be float32, one weight a stream")
+    if rows is None and n < m:
+        raise KernelError("streams_norm: fewer input rows than output rows")
+    if total is not None and (total.dtype != torch.float32 or total.shape != (m, d) or not total.is_contiguous()):
+        raise KernelError("streams_norm: total must be contiguous float32 [m, d]")
+    _i32(rows, "rows", m)
+    lib = _lib("streams")
+    _launch(lib, lib.gb_streams_norm, _p(X), X.stride(0), S, _p(w_in), _p(gamma), dtype_code(gamma), _p(rows), _p(out),
+            dtype_code(out), _p(total), m, d, float(eps), _stream())
+
+
+def streams_mix(X: torch.Tensor, mix: torch.Tensor, w_out: torch.Tensor, y: torch.Tensor) -> None:
+    """In place, all streams at once from the old ones: X[t] = sum_s mix[s, t] X[s] + w_out[t] y."""
+    _dev(X, mix, w_out, y)
+    S, n, d = _streams(X, "streams_mix")
+    if y.dtype != torch.float32 or y.shape != (n, d) or not y.is_contiguous():
+        raise KernelError("streams_mix: y must be contiguous float32 [n, d]")
+    if mix.dtype != torch.float32 or mix.shape != (S, S) or not mix.is_contiguous() or w_out.dtype != torch.float32 \
+            or w_out.numel() != S or not w_out.is_contiguous():
+        raise KernelError("streams_mix: mix must be float32 [streams, streams] and w_out float32 [streams]")
+    lib = _lib("streams")
+    _launch(lib, lib.gb_streams_mix, _p(X), X.stride(0), S, _p(mix), _p(w_out), _p(y), n * d, _stream())
+
+
+# ------------------------------------------------------------------- linear attention
+LINEAR_MAX_KEY_DIM = 256   # linear_attention.hip: a lane holds at most 32 rows of its column of the state
+
+
+def _f32_rows(t: torch.Tensor, shape, what: str) -> None:
+    if t.dtype != torch.float32 or tuple(t.shape) != tuple(shape) or not t.is_contiguous():
+        raise KernelError(f"{what} must be contiguous float32 {tuple(shape)}")
+
+
+def retention_prep(proj: torch.Tensor, q_off: int, k_off: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                   q32: torch.Tensor, k32: torch.Tensor, n_heads: int, key_dim: int, rot: int, k_scale: float) -> None:
+    """q32, k32 (float32 [n, heads * key_dim]) from the query and key heads at columns ``q_off`` and ``k_off`` of the
+    projection's rows: the first ``rot`` dimensions of each head turned in rotate-half pairs by the rows' angles
+    (``cos``, ``sin`` float32 [n, rot / 2]), the keys then times ``k_scale``."""
+    _dev(proj, cos, sin, q32, k32)
+    n = proj.shape[0]
+    stride = _rows(proj, "proj")
+    _f32_rows(q32, (n, n_heads * key_dim), "q32")
+    _f32_rows(k32, (n, n_heads * key_dim), "k32")
+    if rot:
+        for t in (cos, sin):
+            if t is None or t.dtype != torch.float32 or not t.is_contiguous() or t.shape[1] != rot // 2 or t.shape[0] < n:
+                raise KernelError("retention_prep: cos/sin must be contiguous float32 [n, rot / 2]")
+    if max(q_off, k_off) + n_heads * key_dim > proj.shape[1]:
+        raise KernelError("retention_prep: the heads lie beyond the projection's rows")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_retention_prep, _p(proj), dtype_code(proj), stride, int(q_off), int(k_off), _p(cos) if rot else None,
+            _p(sin) if rot else None, _p(q32), _p(k32), n, n_heads, key_dim, int(rot), float(k_scale), _stream())
+
+
+def gla_prep(proj: torch.Tensor, q_off: int, k_off: int, low_off: int, a2: torch.Tensor, a2_bias: Optional[torch.Tensor],
+             q32: torch.Tensor, k32: torch.Tensor, decay: torch.Tensor, q_scale: float, tau: float) -> None:
+    """q32 = q * q_scale, k32 = k, decay = sigmoid(z)^(1/tau) with z = a2 . low + a2_bias, all float32 [n, width], from
+    the projection's rows (queries, keys and the low-rank rows at the given columns; ``a2`` [width, rank] in the
+    projection's type)."""
+    _dev(proj, a2, a2_bias, q32, k32, decay)
+    n = proj.shape[0]
+    stride = _rows(proj, "proj")
+    width, rank = a2.shape
+    for t, what in ((q32, "q32"), (k32, "k32"), (decay, "decay")):
+        _f32_rows(t, (n, width), what)
+    if a2.dtype != proj.dtype or not a2.is_contiguous():
+        raise KernelError("gla_prep: a2 must be contiguous and of the projection's type")
+    if a2_bias is not None:
+        _f32_rows(a2_bias, (width,), "a2_bias")
+    if max(q_off, k_off) + width > proj.shape[1] or low_off + rank > proj.shape[1]:
+        raise KernelError("gla_prep: the heads lie beyond the projection's rows")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_gla_prep, _p(proj), dtype_code(proj), stride, int(q_off), int(k_off), int(low_off), _p(a2),
+            _p(a2_bias), _p(q32), _p(k32), _p(decay), n, width, rank, float(q_scale), 1.0 / float(tau), _stream())
+
+
+def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torch.Tensor, state: torch.Tensor, ctx,
+                n_heads: int, key_dim: int, value_dim: int, decay: Optional[torch.Tensor] = None,
+                head_decay: Optional[torch.Tensor] = None) -> None:
+    """The recurrence S <- diag(a) S + k v^T, o = S^T q over each request's rows of the step, in their order, from the
+    state in the request's slot (empty for a request at position 0) and back into it.  ``decay`` float32
+    [n, heads * key_dim] (a decay a key channel and token) or ``head_decay`` float32 [heads]; ``v`` rows of
+    heads * value_dim in the activations' type (may be a view into wider rows); ``out`` float32 [n, heads * value_dim];
+    ``state`` float32 [slots, heads, value_dim, key_dim]."""
+    _dev(q32, k32, v, out, state, decay, head_decay)
+    n = q32.shape[0]
+    _f32_rows(q32, (n, n_heads * key_dim), "q32")
+    _f32_rows(k32, (n, n_heads * key_dim), "k32")
+    _f32_rows(out, (n, n_heads * value_dim), "out")
+    if (decay is None) == (head_decay is None):
+        raise KernelError("linear_scan: a decay a head or a decay a key channel, one of the two")
+    if decay is not None:
+        _f32_rows(decay, (n, n_heads * key_dim), "decay")
+    else:
+        _f32_rows(head_decay, (n_heads,), "head_decay")
+    if v.shape != (n, n_heads * value_dim):
+        raise KernelError("linear_scan: v must be [n, heads * value_dim]")
+    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, value_dim, key_dim):
+        raise KernelError("linear_scan: state must be contiguous float32 [slots, heads, value_dim, key_dim]")
+    if key_dim > LINEAR_MAX_KEY_DIM:
+        raise KernelError(f"linear_scan: a key size of {key_dim} is above {LINEAR_MAX_KEY_DIM}")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_linear_scan, _p(q32), _p(k32), _p(decay), _p(head_decay), _p(v), dtype_code(v), _rows(v, "v"), _p(out),
+            _p(state), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0), _p(ctx.state_slots), ctx.num_seqs, n_heads, key_dim,
+            value_dim, _stream())
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor, n_heads: int,
+                   value_dim: int, eps: float) -> None:
+    """out[t, h] = weight * o[t, h] / sqrt(mean(o[t, h]^2) + eps) * silu(gate[t, h]) (``weight`` float32 [value_dim] shared
+    by the heads, or None); o float32, gate and out in the activations' type."""
+    _dev(o, gate, weight, out)
+    n = o.shape[0]
+    _f32_rows(o, (n, n_heads * value_dim), "o")
+    if gate.shape != (n, n_heads * value_dim) or out.shape != (n, n_heads * value_dim) or gate.dtype != out.dtype \
+            or not out.is_contiguous():
+        raise KernelError("head_norm_gate: gate and out must be [n, heads * value_dim] of one type, out contiguous")
+    if weight is not None:
+        _f32_rows(weight, (value_dim,), "weight")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_head_norm_gate, _p(o), _p(gate), dtype_code(out), _rows(gate, "gate"), _p(weight), _p(out), n, n_heads,
+            value_dim, float(eps), _stream())
 
 
 # ------------------------------------------------------------------------ products
@@ -627,20 +842,25 @@ PLAIN_SPLIT_MAX_PAIRS = 1024   # (token, head) pairs up to which a step of long 
 PLAIN_GROUP_MIN_ROWS = 64
 
 
-def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size: int, max_context: int) -> int:
+def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size: int, max_context: int,
+                                 keep_first: int = 0) -> int:
     """Floats of workspace with which ``attention_plain`` spreads the chunks of long contexts over workgroups, or 0
     where it would not: many (token, head) pairs fill the chip by themselves, and a context of one chunk has
     nothing to spread.  The bits of the result are the same either way."""
     if n * n_heads > PLAIN_SPLIT_MAX_PAIRS or max_context <= 256:
         return 0
-    return int(_lib("attention_plain").gb_attention_plain_split_floats(n, n_heads, head_dim, page_size, max_context))
+    f = _lib("attention_plain").gb_attention_plain_split_floats
+    f.restype = C.c_longlong
+    return int(f(n, n_heads, head_dim, page_size, max_context, int(keep_first)))
 
 
 def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
                     tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
                     scale: float, window: int = 0, workspace: Optional[torch.Tensor] = None, max_context: int = 0,
-                    grouped: bool = False) -> None:
+                    grouped: bool = False, keep_first: int = 0) -> None:
     """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows.
+    ``window`` > 0: a token at position p reads keys p - window + 1 .. p, and with ``keep_first`` also keys
+    0 .. keep_first - 1 wherever the window has moved past them.
     ``workspace`` (float32, ``attention_plain_split_floats`` elements) with ``max_context`` (at least the most keys a
     token of the step reads): a workgroup a chunk of 256 keys and a second kernel that merges them, for steps of few
     tokens with long contexts; the same bits as without.  ``grouped`` (without a workspace): a workgroup takes eight
@@ -664,17 +884,18 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     lib = _lib("attention_plain")
     _launch(lib, lib.gb_attention_plain, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
                                        _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
-                                       n_heads, nkv, hd, page_size, float(scale), int(window), _p(workspace),
-                                       workspace.numel() if workspace is not None else 0, int(max_context),
+                                       n_heads, nkv, hd, page_size, float(scale), int(window), int(keep_first),
+                                       _p(workspace), workspace.numel() if workspace is not None else 0, int(max_context),
                                        1 if grouped else 0, _stream())
 
 
-def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int) -> bool:
+def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int, keep_first: int = 0) -> bool:
     """Whether the matrix-core attention kernels take this layer: bfloat16 pages, a head size that is
-    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys."""
+    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys, no kept first
+    keys beside a window."""
     _, nkv, n_pieces, page, piece = k_pages.shape
     hd = n_pieces * piece
-    return (k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
+    return (keep_first == 0 and k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
             and n_heads // nkv <= 16 and page >= 16 and page & (page - 1) == 0)
 
 

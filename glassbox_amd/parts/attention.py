@@ -20,23 +20,27 @@ from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding,
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, n_heads: int, scale: float,
-                    window: int) -> None:
-    """Attention of every row of the step over its request's pages.
+                    window: int, keep_first: int = 0) -> None:
+    """Attention of every row of the step over its request's pages.  ``window`` > 0: a token reads the last so many
+    keys up to its own, and with ``keep_first`` the request's first so many keys as well, wherever they lie.
 
     float32 always takes the plain kernel.  bfloat16 takes the tuned kernels where they apply: requests with
     one row go to the split-context decode kernel, longer portions to the matrix-core prefill kernel; a step
     with ``ctx.tuned`` off takes the plain kernel throughout."""
-    if ctx.dtype == torch.float32 or not ctx.tuned or not ops.tuned_attention_supports(cache.k_pages, n_heads, window):
+    if (ctx.dtype == torch.float32 or not ctx.tuned
+            or not ops.tuned_attention_supports(cache.k_pages, n_heads, window, keep_first)):
         longest = int(ctx.host["max_context"])
         _, _, n_pieces, page_size, piece = cache.k_pages.shape
         tables = ctx.tables[cache.group]
 
         def rows(a, b, grouped):
             # few tokens with long contexts (a decode step): a workgroup a chunk of the context, merged by a second kernel
-            floats = 0 if grouped else ops.attention_plain_split_floats(b - a, n_heads, n_pieces * piece, page_size, longest)
+            floats = 0 if grouped else ops.attention_plain_split_floats(b - a, n_heads, n_pieces * piece, page_size, longest,
+                                                                        keep_first)
             ws = ctx.buffer("attention_plain_parts", (floats,), torch.float32) if floats else None
             ops.attention_plain(q[a:b], out[a:b], ctx.positions[a:b], ctx.tok_seq[a:b], tables, cache.k_pages, cache.v_pages,
-                                n_heads, scale, window, workspace=ws, max_context=longest, grouped=grouped)
+                                n_heads, scale, window, workspace=ws, max_context=longest, grouped=grouped,
+                                keep_first=keep_first)
 
         # the rows of requests with one token come first; many rows of prompt portions go eight rows a workgroup
         n, n_decode = q.shape[0], ctx.host["n_decode"]
@@ -145,3 +149,76 @@ class PagedAttention(Mixer):
         ops.gemm(att, self.wo, residual, accumulate=True, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.q_dim))
         return handed_on
+
+
+class TiedValueAttention(Mixer):
+    """Grouped-query attention whose values are its keys: there is no value projection, and a key head as projected
+    (bias included, before any norm) is the value head.  Options, each a constructor argument: biases on the query,
+    key and output projections; an RMS norm of every query and key head over its dimensions, with a weight for the
+    queries and one for the keys that the heads share; the scale of the scores; a window of the last ``window`` keys,
+    with the request's first ``keep_first`` keys visible for good.  Positions do not enter the scores.
+
+    Tensors: ``q``, ``k``, ``o`` (and ``q.b``, ``k.b``, ``o.b``; ``q.norm``, ``k.norm``)."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: Optional[float] = None,
+                 window: int = 0, keep_first: int = 0, bias: bool = True, qk_norm: bool = True, eps: float = 1e-5):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key heads")
+        if keep_first and not window:
+            raise ValueError("kept first keys go with a window")
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.window, self.keep_first = int(window), int(keep_first)
+        self.bias, self.qk_norm, self.eps = bool(bias), bool(qk_norm), float(eps)
+        self.q_dim, self.kv_dim = n_heads * head_dim, n_kv_heads * head_dim
+        self.cache_spec = CacheSpec(n_kv_heads, head_dim, WINDOW if window > 0 else FULL, self.window, self.keep_first)
+        self.wqk = self.wo = self.bias_q = self.bias_k = self.bias_o = self.norm_q = self.norm_k = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = {"q": TensorSpec((self.q_dim, self.width)), "k": TensorSpec((self.kv_dim, self.width)),
+                 "o": TensorSpec((self.width, self.q_dim))}
+        if self.bias:
+            specs.update({"q.b": TensorSpec((self.q_dim,), kind="f32", init="normal"),
+                          "k.b": TensorSpec((self.kv_dim,), kind="f32", init="normal"),
+                          "o.b": TensorSpec((self.width,), kind="f32", init="normal")})
+        if self.qk_norm:
+            specs.update({"q.norm": TensorSpec((self.head_dim,), kind="f32", init="ones"),
+                          "k.norm": TensorSpec((self.head_dim,), kind="f32", init="ones")})
+        return specs
+
+    def load(self, tensors):
+        self.wqk = torch.cat([tensors["q"], tensors["k"]], 0)   # one product computes both
+        self.wo = tensors["o"].contiguous()
+        if self.bias:
+            self.bias_q, self.bias_k, self.bias_o = (tensors[n].contiguous() for n in ("q.b", "k.b", "o.b"))
+        if self.qk_norm:
+            self.norm_q, self.norm_k = tensors["q.norm"].contiguous(), tensors["k.norm"].contiguous()
+
+    def streamed_matrices(self):
+        return [self.wqk, self.wo]
+
+    def problems(self, dtype, page_size):
+        out = needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "heads * dim", self.q_dim)
+        if self.head_dim > ops.MAX_HEAD_DIM:
+            out.append(("dim", f"{self.head_dim} is above {ops.MAX_HEAD_DIM}, the largest head the attention kernels take"))
+        return out
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        if cache is None or cache.k_pages is None:
+            raise ValueError("TiedValueAttention needs a layer cache with pages")
+        n = h.shape[0]
+        qk = ctx.buffer("qk", (n, self.q_dim + self.kv_dim), ctx.dtype)
+        ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
+        slots = ctx.slots[cache.group] if cache.writable else None
+        ops.qk_norm_store(qk, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, slots,
+                          cache.k_pages if slots is not None else None, cache.v_pages if slots is not None else None,
+                          self.n_heads, self.n_kv_heads, self.head_dim)
+        att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
+        paged_attention(ctx, qk[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window, self.keep_first)
+        ops.gemm(att, self.wo, residual, accumulate=not store, workspace=split_workspace(ctx, n, self.width, self.q_dim))
+        if self.bias_o is not None:
+            ops.add_bias(residual, self.bias_o)

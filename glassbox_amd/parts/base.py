@@ -48,7 +48,8 @@ class TensorSpec:
     """A tensor a part needs.  ``kind`` decides its type on the device:
     'matrix' follows the compute type (bfloat16 or float32); 'vector' keeps 32-bit storage if the
     file has it and is bfloat16 otherwise (float32 in the 32-bit path); 'f32' is always float32;
-    'int' becomes int32.  ``init`` is what the random-weights mode draws: 'normal', 'ones', 'zeros'."""
+    'int' becomes int32.  ``init`` is what the random-weights mode draws: 'normal', 'ones', 'zeros', 'eye'.  A size of
+    -1 is one that only the checkpoint's tensor gives (no key of config.json does); the part reads it in ``load``."""
     shape: Tuple[int, ...]
     kind: str = "matrix"
     init: str = "normal"
@@ -56,15 +57,18 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class CacheSpec:
-    """Paged keys and values of one layer.  kind FULL keeps every position, WINDOW the last ``window``."""
+    """Paged keys and values of one layer.  kind FULL keeps every position, WINDOW the last ``window`` and, with
+    ``keep_first``, the first so many as well."""
     num_kv_heads: int
     head_dim: int
     kind: int = FULL
     window: int = 0
+    keep_first: int = 0
 
     @property
-    def group_key(self) -> Tuple[int, int]:
-        return (self.kind, self.window if self.kind == WINDOW else 0)
+    def group_key(self) -> Tuple[int, int, int]:
+        windowed = self.kind == WINDOW
+        return (self.kind, self.window if windowed else 0, self.keep_first if windowed else 0)
 
 
 @dataclass(frozen=True)

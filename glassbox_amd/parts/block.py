@@ -63,3 +63,26 @@ class PreNormBlock(Block):
         if spec is not None:
             return self.ffn.forward(ctx, x, x, norm=spec, **more)
         return self.ffn.forward(ctx, self.ffn_norm.forward(ctx, x), x, **more)
+
+
+class MixerOnlyBlock(Block):
+    """A layer without a feed-forward: norm, mixer, add."""
+    replayable = True
+    taped = True
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, names=("norm1", "mix")):
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.names = tuple(names)
+
+    def children(self) -> Dict[str, Part]:
+        return dict(zip(self.names, (self.mixer_norm, self.mixer)))
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return self.mixer.cache_spec
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return self.mixer.state_spec
+
+    def forward(self, ctx, x, cache: Optional[LayerCache]):
+        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, x), x, cache)
+        return None

@@ -14,8 +14,8 @@ from .base import Part, TensorSpec, needs_multiple_of_8
 class Embedding(Part):
     replayable = True
 
-    def __init__(self, vocab: int, width: int):
-        self.vocab, self.width = vocab, width
+    def __init__(self, vocab: int, width: int, scale: float = 1.0):
+        self.vocab, self.width, self.scale = vocab, width, float(scale)
         self.table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -25,15 +25,16 @@ class Embedding(Part):
         self.table = tensors["weight"].contiguous()
 
     def forward(self, ctx, out):
-        ops.embed(self.table, ctx.token_ids, out)
+        """``out`` [n, width], or [streams, n, width]: every stream starts as the embedding."""
+        ops.embed(self.table, ctx.token_ids, out, self.scale)
 
 
 class LMHead(Part):
-    """logits = rows . W^T in float32.  ``tied_to`` names an Embedding whose table is the head."""
+    """logits = rows . W^T (times ``scale``) in float32.  ``tied_to`` names an Embedding whose table is the head."""
     replayable = True
 
-    def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None):
-        self.vocab, self.width, self.tied_to = vocab, width, tied_to
+    def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None, scale: float = 1.0):
+        self.vocab, self.width, self.tied_to, self.scale = vocab, width, tied_to, float(scale)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -58,4 +59,6 @@ class LMHead(Part):
         """``prepared``: a PreNormed whose rows these are: the product scales its result by the norm's factor."""
         logits = ctx.buffer("logits", (rows.shape[0], self.vocab), torch.float32)
         ops.gemm(rows, self.matrix(), logits, rms_parts=prepared.as_gemm_arg() if prepared is not None else None)
+        if self.scale != 1.0:
+            ops.scale_rows(logits, self.scale)
         return logits

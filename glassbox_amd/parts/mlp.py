@@ -36,11 +36,13 @@ class SwiGLU(FeedForward):
 
     accepts_fused_norm = True
     accepts_emit_norm = True
+    accepts_store = True
 
-    def forward(self, ctx, h, residual, norm=None, emit=None):
+    def forward(self, ctx, h, residual, norm=None, emit=None, store: bool = False):
         """``norm=(gamma, eps)``: h is the un-normed float32 residual and the first product norms it;
         ``norm=PreNormed``: the product before has done most of that.  ``emit=(gamma, eps)``: the down
-        projection may prepare the norm that reads the residual next (returns a PreNormed or Normed if it did)."""
+        projection may prepare the norm that reads the residual next (returns a PreNormed or Normed if it did).
+        ``store``: the rows are written to ``residual`` (float32) instead of added."""
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
         if isinstance(norm, PreNormed):
@@ -57,7 +59,7 @@ class SwiGLU(FeedForward):
             gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
             ops.gemm(h, self.w_gate_up, gate_up)
             ops.silu_mul(gate_up, act)
-        target, handed_on = emit_target(ctx, n, self.width, self.intermediate, emit, "ffn")
-        ops.gemm(act, self.w_down, residual, accumulate=True, emit=target,
+        target, handed_on = emit_target(ctx, n, self.width, self.intermediate, None if store else emit, "ffn")
+        ops.gemm(act, self.w_down, residual, accumulate=not store, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.intermediate))
         return handed_on

@@ -33,8 +33,12 @@ class DecoderModel(Part):
 
     def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
                  final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
-                 ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None, sources=None):
+                 ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None, sources=None,
+                 streams: Optional[int] = None):
         self.config = config
+        #: None: one residual [n, width]; a number: the residual is so many streams, [streams, n, width], which the
+        #: embedding fills alike and the blocks and the final norm take as such (parts.streams)
+        self.streams = streams
         #: where the checkpoint keeps a tensor that it names or cuts otherwise than the parts do: a mapping, or a
         #: function, from the model's tensor name to the checkpoint's name or to (name, first row, last row) of a
         #: tensor that holds several stacked by rows; None for a tensor of the same name (weights.loader)
@@ -94,7 +98,8 @@ class DecoderModel(Part):
     # the step ---------------------------------------------------------------------
     def forward(self, ctx, caches: Sequence[LayerCache]) -> torch.Tensor:
         """Runs the tokens of ``ctx`` through every scheduled layer; logits [wanted, vocab] float32."""
-        x = ctx.buffer("x", (ctx.n, self.width), torch.float32)
+        shape = (ctx.n, self.width) if self.streams is None else (self.streams, ctx.n, self.width)
+        x = ctx.buffer("x", shape, torch.float32)
         self.embedding.forward(ctx, x)
         pre = None   # what the block before prepared of this block's first norm
         if self._taped is None:

@@ -124,6 +124,12 @@ def checkpoint_layout(model) -> Tuple[Dict[str, Source], Dict[str, Tuple[int, ..
     return sources, shapes
 
 
+def _fits(actual: Tuple[int, ...], declared: Tuple[int, ...]) -> bool:
+    """Whether a tensor of the file has the declared shape; a declared size of -1 is whatever the file has (a size
+    that no key of config.json gives: the part reads it from the tensor)."""
+    return len(actual) == len(declared) and all(d == -1 or d == a for a, d in zip(actual, declared))
+
+
 def load_weights(model, path: str, dtype: torch.dtype, device) -> None:
     try:
         f = SafetensorsFile(path)
@@ -134,7 +140,7 @@ def load_weights(model, path: str, dtype: torch.dtype, device) -> None:
     have = set(f.names())
     missing = sorted(n for n in shapes if n not in have)
     unexpected = sorted(n for n in have if n not in shapes and n not in getattr(model, "ignorable", ()))
-    wrong = sorted((n, f.shape(n), shapes[n]) for n in shapes if n in have and tuple(f.shape(n)) != shapes[n])
+    wrong = sorted((n, f.shape(n), shapes[n]) for n in shapes if n in have and not _fits(tuple(f.shape(n)), shapes[n]))
     if missing or unexpected or wrong:
         lines = [f"{path} does not fit the model {type(model.config).__name__}:"]
         if missing:
@@ -180,8 +186,14 @@ def random_tensors(model, seed: int, std: float = 0.02, norm_init: str = "ones",
     gen.manual_seed(seed)
     out = {}
     for name, spec in sorted(model.named_specs()):
+        if any(s < 0 for s in spec.shape):
+            raise WeightError(f"{name}: a size that only a checkpoint's tensor gives; random weights need it stated")
         if spec.kind == "int":
             t = torch.zeros(spec.shape, dtype=torch.int32, device=device)
+        elif spec.init == "eye":
+            t = torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device)
+            if norm_init == "uniform":   # off-diagonal weights too, so that a transposed matrix shows
+                t = t + (torch.rand(spec.shape, generator=gen, device=device, dtype=torch.float32) - 0.5) * 0.5
         elif spec.init == "ones":
             if norm_init == "uniform":
                 t = torch.rand(spec.shape, generator=gen, device=device, dtype=torch.float32) + 0.5
