@@ -43,6 +43,19 @@ int gb_attention_decode_bf16_static(const void* q, int q_stride, void* out, int 
                                     int n_decode, int nh, int nkv, int hd, int page_size, float scale, int window,
                                     int chunk, int max_context, hipStream_t stream);
 
+// The two kernels with kept first keys beside the window: keys 0 .. keep_first-1 of a request are read by every
+// later token, wherever its window lies (keep_first = 0: the entry points above and below).
+int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
+                                  const int32_t* positions, const int32_t* tables, int table_stride, const void* k_pages,
+                                  const void* v_pages, int n_decode, int nh, int nkv, int hd, int page_size, float scale,
+                                  int window, int keep_first, int chunk, int max_context, hipStream_t stream);
+int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
+                                   const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs, int max_q_len,
+                                   int max_context, const int32_t* tables, int table_stride, const void* k_pages,
+                                   const void* v_pages, int nh, int nkv, int hd, int page_size, float scale, int window,
+                                   int keep_first, int first_row, int n_rows, float* part_ws, long long part_floats,
+                                   hipStream_t stream);
+
 int gb_attention_prefill_parts(int max_q_len, int max_context, int nh, int n_seqs, int hd);
 
 int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,

@@ -153,7 +153,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
                                                             float* __restrict__ ws_ml, const int32_t* __restrict__ positions,
                                                             const int32_t* __restrict__ tables, int table_stride,
                                                             const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh,
-                                                            int nkv, int P, float scale, int window, int chunk, int splits) {
+                                                            int nkv, int P, float scale, int window, int keep, int chunk,
+                                                            int splits) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
   extern __shared__ float decode_lds[];
   const int s = blockIdx.z, kvh = blockIdx.y, split = blockIdx.x;
@@ -164,7 +165,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   const int pos = positions[s];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int c0 = split * chunk;
-  if (c0 > pos || c0 + chunk <= lo) return;  // this chunk holds no key of the request
+  const int kept = min(keep, lo);            // keys 0 .. kept-1 are read although the window has passed them
+  if (c0 > pos || (c0 + chunk <= lo && c0 >= kept)) return;  // this chunk holds no key of the request
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15;
   const int32_t* table = tables + (size_t)s * table_stride;
@@ -180,6 +182,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   const int col_lo = col < G ? lo : 1, col_hi = col < G ? pos : 0;
   const int end = min(c0 + chunk, pos + 1);
   for (int kb = c0 + wave * 64; kb < end; kb += 64 * WAVES) {
+    // the kept first keys of these 64, then those inside the window (a tile can hold both kinds)
+    if (kb < kept) attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane);
     if (kb + 64 <= lo) continue;
     attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane);
   }
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                                                             bf16* __restrict__ out, int out_stride,
                                                             const int32_t* __restrict__ positions, int nh, int hd, int window,
-                                                            int chunk, int splits) {
+                                                            int keep, int chunk, int splits) {
   constexpr int EARLY = 4;           // partial results a thread asks for before it knows their weights
   __shared__ float sm_f[256];        // chunk k's weight exp(m_k - M)
   __shared__ float sm_part[256];     // [group][dimension]
@@ -241,19 +245,23 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restr
   const int s = blockIdx.x / nh, head = blockIdx.x % nh, tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int pos = positions[s];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int first = lo / chunk, last = pos / chunk, count = last - first + 1;  // at most 256 chunks hold keys
-  const size_t base = ((size_t)s * nh + head) * splits + first;
+  // the chunks that hold keys: those of the kept first keys that lie before the window's first chunk, then the window's
+  const int first = lo / chunk, last = pos / chunk;
+  const int early_chunks = min((min(keep, lo) + chunk - 1) / chunk, first);
+  const int count = early_chunks + last - first + 1;  // at most 256 chunks hold keys
+  const size_t base0 = ((size_t)s * nh + head) * splits;
+  auto cell_of = [&](int k) { return base0 + (k < early_chunks ? k : first + (k - early_chunks)); };
   const int groups = 256 / hd;  // hd <= 128: at least two
   const int d = tid % hd, group = tid / hd;
   float mine = -INFINITY, mine_l = 0.f, early[EARLY];
   if (tid < count) {
-    mine = ws_ml[(base + tid) * 2];
-    mine_l = ws_ml[(base + tid) * 2 + 1];
+    mine = ws_ml[cell_of(tid) * 2];
+    mine_l = ws_ml[cell_of(tid) * 2 + 1];
   }
 #pragma unroll
   for (int i = 0; i < EARLY; ++i) {
     const int k = group + i * groups;
-    early[i] = (group < groups && k < count) ? ws_acc[(base + k) * hd + d] : 0.f;
+    early[i] = (group < groups && k < count) ? ws_acc[cell_of(k) * hd + d] : 0.f;
   }
   float top = mine;
 #pragma unroll
@@ -275,7 +283,7 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restr
       const int k = group + i * groups;
       if (k < count) val += early[i] * sm_f[k];
     }
-    for (int k = group + EARLY * groups; k < count; k += groups) val += ws_acc[(base + k) * hd + d] * sm_f[k];
+    for (int k = group + EARLY * groups; k < count; k += groups) val += ws_acc[cell_of(k) * hd + d] * sm_f[k];
   }
   sm_part[tid] = val;
   __syncthreads();
@@ -315,9 +323,10 @@ struct PageSource {
   const int32_t* __restrict__ table;
   int nkv, kvh, shift;  // pages of 1 << shift keys
   int tlo, thi;         // groups of 16 keys outside [tlo, thi] are redirected into it (their keys are masked anyway)
+  int keep16 = 0;       // but for the groups below this key: the kept first keys, whose pages a window leaves in place
   // offset, in elements of a page array of one kv head, of the page and slot that hold key k
   __device__ __forceinline__ size_t page_of(int k, int* slot) const {
-    const int kc = min(max(k, tlo), thi);
+    const int kc = min(k < keep16 ? k : max(k, tlo), thi);
     *slot = kc & ((1 << shift) - 1);
     return ((size_t)table[kc >> shift] * nkv + kvh);
   }
@@ -369,7 +378,8 @@ template <int HD, int QB, int ACT, int T = 2>
 __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32x16 (&acc)[QB][(HD + 31) / 32],
                                              const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[T][HD / 16],
                                              bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int next,
-                                             const int (&lo)[QB], const int (&hi)[QB], bool mask, float c, int lane) {
+                                             const int (&lo)[QB], const int (&hi)[QB], bool mask, float c, int lane,
+                                             int keep = 0) {
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
   constexpr int LAST = (ACT & 2) ? 1 : 0;
   const int g = lane >> 5;
@@ -400,7 +410,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = kbase + 32 * t + 16 * (r >> 3) + 8 * g + 4 * ((r >> 2) & 1) + (r & 3);
-          if (key < lo[qb] || key > hi[qb]) s[t][r] = -INFINITY;
+          if ((key < lo[qb] && key >= keep) || key > hi[qb]) s[t][r] = -INFINITY;
         }
     }
     float mx = -INFINITY;
@@ -570,8 +580,9 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
                                                       int seq_base, const int32_t* __restrict__ tables, int table_stride,
                                                       const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh, int nkv,
-                                                      int page_shift, float scale, int window, float* __restrict__ part_acc,
-                                                      float* __restrict__ part_ml, int parts, int first_row, int n_rows) {
+                                                      int page_shift, float scale, int window, int keep,
+                                                      float* __restrict__ part_acc, float* __restrict__ part_ml, int parts,
+                                                      int first_row, int n_rows) {
   // parts > 1: `parts` workgroups share a group's pairs, taking the tiles of keys in turn like the waves of a pair
   // do; each writes its sums to part_acc / part_ml (rows counted from first_row), and prefill_parts_kernel adds them.
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
@@ -598,7 +609,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
   const int col = lane & 31, g = lane >> 5;
   const int p0 = pos0[seq];
   const int kvh = head / (nh / nkv);
-  PageSource src{kp, vp, tables + (size_t)seq * table_stride, nkv, kvh, page_shift, 0, 0};
+  PageSource src{kp, vp, tables + (size_t)seq * table_stride, nkv, kvh, page_shift, 0, 0, (keep + 15) & ~15};
   const size_t row0 = (size_t)q_start[seq];
   const float c = scale * 1.4426950408889634f;
   constexpr int T = QB == 2 ? 2 : 1;  // tiles of 32 keys a step: with one block live at a time (the larger head
@@ -644,8 +655,11 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
     src.thi = end & ~15;
     // the tiles of 64 keys in order: both blocks as far as the earlier one's keys reach (with a window the later
     // one may see none of them yet: they are masked), then, with a window after a gap, the later block alone
+    // with kept first keys: their tiles of 64 first (as far as they lie before the window's first tile), both blocks live
+    const int win0 = range[0].first & ~63, kept_end = min((keep + 63) & ~63, win0);
     auto after = [&](int kb) {
       int next = kb + 64;
+      if (kb < kept_end && next >= kept_end) next = win0;
       if (has_second && kb <= range[0].last && next > range[0].last && next + 63 < range[1].first) next = range[1].first & ~63;
       return next;
     };
@@ -653,7 +667,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       for (int i = 0; i < SPLIT * parts; ++i) kb = after(kb);
       return kb;
     };
-    int kb = range[0].first & ~63;
+    int kb = kept_end > 0 ? 0 : win0;
     for (int i = 0; i < part * SPLIT + half; ++i) kb = after(kb);
     if (!works) kb = end + 1;  // (a pair beyond the request's last block only goes to the barriers)
     load_keys<HD, T>(kf, src, kb, lane);
@@ -662,18 +676,18 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       while (kb <= range[0].last) {
         const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
-        attend64_q32<HD, 2, 3>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane);
+        attend64_q32<HD, 2, 3>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep);
         kb = next;
       }
       while (kb <= range[1].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane);
+        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep);
         kb = next;
       }
     } else {
       while (kb <= range[0].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane);
+        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep);
         kb = next;
       }
     }
@@ -714,12 +728,16 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       src.tlo = range.first & ~15;
       src.thi = range.last & ~15;
       constexpr int SPAN = 32 * T;  // the waves of the pair take the steps of SPAN keys in turn
-      const int kb0 = (range.first & ~(SPAN - 1)) + (part * SPLIT + half) * SPAN, stride = SPAN * SPLIT * parts;
-      load_keys<HD, T>(kf, src, kb0, lane);
-      load_values<HD, T>(vf, src, kb0, lane);
-      for (int kb = kb0; kb <= range.last; kb += stride)
-        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, kb, kb + stride, lo, hi, !range.unmasked(kb, SPAN), c,
-                                  lane);
+      // step i of the block: the steps over the kept first keys (as far as they lie before the window's first step),
+      // then the window's
+      const int win0 = range.first & ~(SPAN - 1), kept_steps = min((keep + SPAN - 1) & ~(SPAN - 1), win0) / SPAN;
+      auto key_of = [&](int i) { return i < kept_steps ? i * SPAN : win0 + (i - kept_steps) * SPAN; };
+      const int i0 = part * SPLIT + half, stride = SPLIT * parts;
+      load_keys<HD, T>(kf, src, key_of(i0), lane);
+      load_values<HD, T>(vf, src, key_of(i0), lane);
+      for (int i = i0; key_of(i) <= range.last; i += stride)
+        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
+                                  !range.unmasked(key_of(i), SPAN), c, lane, keep);
       if constexpr (SPLIT > 1) {
         hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);
         if (half != 0) continue;
@@ -743,11 +761,13 @@ extern "C" int gb_attention_supported_head_size(int hd) { return hd >= 16 && hd 
 
 // q, out: rows 0 .. n_decode-1 are the decoding requests (one row each).  ws_acc must hold
 // n_decode*nh*splits*hd floats and ws_ml n_decode*nh*splits*2, with splits = ceil(max_context / chunk).
-extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
-                                        const int32_t* positions, const int32_t* tables, int table_stride,
-                                        const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
-                                        int page_size, float scale, int window, int chunk, int max_context,
-                                        hipStream_t stream) {
+// keep_first > 0 (with a window): keys 0 .. keep_first-1 are read wherever the window has moved past them.
+extern "C" int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
+                                             const int32_t* positions, const int32_t* tables, int table_stride,
+                                             const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
+                                             int page_size, float scale, int window, int keep_first, int chunk,
+                                             int max_context, hipStream_t stream) {
+  GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_decode: kept first keys go with a window");
   GB_REQUIRE(n_decode >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_decode: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_decode: head size %d is not a multiple of 16 up to 128", hd);
   GB_REQUIRE(nh / nkv <= 16, "attention_decode: %d query heads per kv head exceed the 16 columns of a tile", nh / nkv);
@@ -772,11 +792,11 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
     if (waves == 16)                                                                                                        \
       hipLaunchKernelGGL((decode_kernel<HD, 16>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride, \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, chunk, splits);                           \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
     else                                                                                                                    \
       hipLaunchKernelGGL((decode_kernel<HD, 4>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride,  \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, chunk, splits);                           \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
   }
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
@@ -784,10 +804,19 @@ extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, 
   if (splits > 1) {
     GB_REQUIRE(splits <= 256, "attention_decode: %d chunks are more than the 256 the second pass combines", splits);
     hipLaunchKernelGGL(decode_reduce_kernel, dim3(n_decode * nh), dim3(256), 0, stream, (const float*)ws_acc,
-                       (const float*)ws_ml, (bf16*)out, out_stride, positions, nh, hd, window, chunk, splits);
+                       (const float*)ws_ml, (bf16*)out, out_stride, positions, nh, hd, window, keep_first, chunk, splits);
     return launched("attention_decode_reduce");
   }
   return 0;
+}
+
+extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
+                                        const int32_t* positions, const int32_t* tables, int table_stride,
+                                        const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
+                                        int page_size, float scale, int window, int chunk, int max_context,
+                                        hipStream_t stream) {
+  return gb_attention_decode_bf16_keep(q, q_stride, out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages,
+                                       v_pages, n_decode, nh, nkv, hd, page_size, scale, window, 0, chunk, max_context, stream);
 }
 
 // ------------------------------------------------------- decoding without a workspace from the caller
@@ -884,12 +913,14 @@ extern "C" int gb_attention_prefill_parts(int max_q_len, int max_context, int nh
 // max_context the longest context any of them reaches (both only shape the launch).  first_row, n_rows: the rows of
 // q and out that the portions occupy (contiguous); part_ws: float32 workspace of part_floats elements, needed if
 // gb_attention_prefill_parts says so.
-extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
-                                         const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs, int max_q_len,
-                                         int max_context, const int32_t* tables, int table_stride, const void* k_pages,
-                                         const void* v_pages, int nh, int nkv, int hd, int page_size, float scale, int window,
-                                         int first_row, int n_rows, float* part_ws, long long part_floats,
-                                         hipStream_t stream) {
+// keep_first > 0 (with a window): keys 0 .. keep_first-1 are read wherever the window has moved past them.
+extern "C" int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
+                                              const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs,
+                                              int max_q_len, int max_context, const int32_t* tables, int table_stride,
+                                              const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
+                                              float scale, int window, int keep_first, int first_row, int n_rows,
+                                              float* part_ws, long long part_floats, hipStream_t stream) {
+  GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_prefill: kept first keys go with a window");
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
   GB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "attention_prefill: page size %d is not a power of two from 16 up", page_size);
@@ -914,7 +945,8 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
 #define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                                                                                     \
   hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT>), grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, \
                      out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
-                     (const bf16*)v_pages, nh, nkv, page_shift, scale, window, part_acc, part_ml, parts, first_row, n_rows)
+                     (const bf16*)v_pages, nh, nkv, page_shift, scale, window, keep_first, part_acc, part_ml, parts, first_row, \
+                     n_rows)
 #define GB_CASE(HD)                                        \
   if (hd == HD) {                                          \
     if constexpr (HD <= 64) {                              \
@@ -940,6 +972,19 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
   return 0;
 }
 
+extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
+                                         const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs, int max_q_len,
+                                         int max_context, const int32_t* tables, int table_stride, const void* k_pages,
+                                         const void* v_pages, int nh, int nkv, int hd, int page_size, float scale, int window,
+                                         int first_row, int n_rows, float* part_ws, long long part_floats,
+                                         hipStream_t stream) {
+  return gb_attention_prefill_bf16_keep(q, q_stride, out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len,
+                                        max_context, tables, table_stride, k_pages, v_pages, nh, nkv, hd, page_size, scale,
+                                        window, 0, first_row, n_rows, part_ws, part_floats, stream);
+}
+
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_attention_decode_bf16_keep)
+GB_TAPED(gb_attention_prefill_bf16_keep)
 GB_TAPED(gb_attention_decode_bf16)
 GB_TAPED(gb_attention_prefill_bf16)

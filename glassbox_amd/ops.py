@@ -104,6 +104,11 @@ _SIGS = {
         "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                                       _f, _i, _i, _i, _vp, C.c_longlong, _vp],
         "gb_attention_prefill_parts": [_i, _i, _i, _i, _i],
+        # the same two with the number of kept first keys after the window
+        "gb_attention_decode_bf16_keep": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
+                                          _i, _i, _vp],
+        "gb_attention_prefill_bf16_keep": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+                                           _f, _i, _i, _i, _i, _vp, C.c_longlong, _vp],
     },
     "sampling": {
         "gb_argmax": [_vp, _vp, _i, _i, _vp],
@@ -891,11 +896,10 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int, keep_first: int = 0) -> bool:
     """Whether the matrix-core attention kernels take this layer: bfloat16 pages, a head size that is
-    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys, no kept first
-    keys beside a window."""
+    a multiple of 16 up to 128, at most 16 query heads per kv head, pages of 16, 32, 64 ... keys."""
     _, nkv, n_pieces, page, piece = k_pages.shape
     hd = n_pieces * piece
-    return (keep_first == 0 and k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
+    return (k_pages.dtype == torch.bfloat16 and hd % 16 == 0 and 16 <= hd <= 128 and n_heads % nkv == 0
             and n_heads // nkv <= 16 and page >= 16 and page & (page - 1) == 0)
 
 
@@ -915,7 +919,8 @@ def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
     return max(256, -(-chunk // 256) * 256)
 
 
-def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int) -> None:
+def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int,
+                     keep_first: int = 0) -> None:
     """Rows 0..n_decode-1 of the step (requests with a single token), split over their context."""
     n_dec = ctx.host["n_decode"]
     k_pages, v_pages = cache.k_pages, cache.v_pages
@@ -930,6 +935,11 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
     ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
     ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
     lib = _lib("attention_bf16")
+    if keep_first:
+        _launch(lib, lib.gb_attention_decode_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
+                _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_dec, n_heads, nkv, hd, page,
+                float(scale), int(window), int(keep_first), chunk, max_context, _stream())
+        return
     _launch(lib, lib.gb_attention_decode_bf16, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
                                              _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages),
                                              n_dec, n_heads, nkv, hd, page, float(scale), int(window), chunk,
@@ -941,7 +951,8 @@ def _prefill_parts(max_q: int, max_ctx: int, n_heads: int, n_seqs: int, hd: int)
     return int(_lib("attention_bf16").gb_attention_prefill_parts(max_q, max_ctx, n_heads, n_seqs, hd))
 
 
-def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int) -> None:
+def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int,
+                      keep_first: int = 0) -> None:
     """The requests of the step that bring more than one token (they follow the single-token ones)."""
     n_dec, S = ctx.host["n_decode"], ctx.num_seqs
     k_pages, v_pages = cache.k_pages, cache.v_pages
@@ -957,6 +968,12 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     first_row, n_rows = n_dec, q.shape[0] - n_dec
     parts = _prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
     ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
+    if keep_first:
+        _launch(lib, lib.gb_attention_prefill_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
+                _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables), tables.stride(0), _p(k_pages),
+                _p(v_pages), n_heads, nkv, hd, page, float(scale), int(window), int(keep_first), first_row, n_rows, _p(ws),
+                ws.numel() if ws is not None else 0, _stream())
+        return
     _launch(lib, lib.gb_attention_prefill_bf16, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                                               _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables),
                                               tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd, page,

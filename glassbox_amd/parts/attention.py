@@ -53,9 +53,9 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, 
         return
     n_decode = ctx.host["n_decode"]
     if n_decode > 0:
-        ops.attention_decode(q, out, ctx, cache, n_heads, scale, window)
+        ops.attention_decode(q, out, ctx, cache, n_heads, scale, window, keep_first)
     if n_decode < ctx.num_seqs:
-        ops.attention_prefill(q, out, ctx, cache, n_heads, scale, window)
+        ops.attention_prefill(q, out, ctx, cache, n_heads, scale, window, keep_first)
 
 
 class PagedAttention(Mixer):

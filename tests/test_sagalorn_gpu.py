@@ -189,6 +189,28 @@ def test_window_with_kept_first_keys_at_its_edges(dtype, window, keep):
         ops.attention_plain(qk[last, :H * hd].contiguous(), out2, _i32(last), _i32([0] * 3), table, k_pages, v_pages, H, scale,
                             window, workspace=ws, max_context=T, keep_first=keep)
         assert torch.equal(out2, out[last])
+    if dtype != torch.bfloat16:
+        return
+    # the matrix-core kernels: the request as one portion, as a portion behind a cached beginning, and single tokens
+    from glassbox_amd.engine.context import Workspace
+    from glassbox_amd.parts.base import LayerCache
+    ws_all, cache = Workspace(torch.device(DEV)), LayerCache(k_pages, v_pages, group=0)
+    for start in (0, 463, T - 2):
+        n = T - start
+        ctx = SimpleNamespace(host={"n_decode": 0, "max_q_len": n, "max_context": T}, num_seqs=1, q_start=_i32([0]),
+                              q_len=_i32([n]), pos0=_i32([start]), tables=[table], buffer=ws_all.buffer)
+        got = torch.zeros(n, H * hd, dtype=dtype, device=DEV)
+        ops.attention_prefill(qk[start:, :H * hd], got, ctx, cache, H, scale, window, keep)
+        err = (got.cpu().to(F64).view(n, H, hd) - want[start:]).abs().amax((1, 2))
+        assert float(err.max()) < tol, ("portion from", start, int(err.argmax()), float(err.max()))
+    rows = [T - 1, min(T - 1, window + keep), max(keep, 1), 5, 300, min(T - 1, window), 0]
+    for chunk_ctx in (T, 2048):   # (the launch's longest context decides how the keys are spread over workgroups)
+        ctx = SimpleNamespace(host={"n_decode": len(rows), "max_context": chunk_ctx}, num_seqs=len(rows), positions=_i32(rows),
+                              tables=[table.expand(len(rows), -1).contiguous()], buffer=ws_all.buffer)
+        got = torch.zeros(len(rows), H * hd, dtype=dtype, device=DEV)
+        ops.attention_decode(qk[rows, :H * hd].contiguous(), got, ctx, cache, H, scale, window, keep)
+        err = (got.cpu().to(F64).view(len(rows), H, hd) - want[rows]).abs().amax((1, 2))
+        assert float(err.max()) < tol, ("single tokens", chunk_ctx, rows[int(err.argmax())], float(err.max()))
 
 
 # ------------------------------------------------------------------------------------------ whole models
