@@ -3,6 +3,12 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
+    python bench.py --design sagalorn [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
+
+``--design sagalorn`` is another measurement with a line of its own: prefill and decode throughput of Sagalorn models
+whose layers have the sizes of the named shapes (a third of the layers each retention, windowed attention with kept
+first keys and gated linear attention, every one with a feed-forward, two residual streams), beside a Llama of the
+same width, heads, feed-forward, vocabulary and number of layers.
 
 A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step``
 (which replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the
@@ -41,6 +47,91 @@ NAMES = {"smollm2-1.7b": "SmolLM2-1.7B shapes", "smollm2-360m": "SmolLM2-360M sh
 PEAK = {"hbm_gbs": 8000.0, "bf16_tflops": 2500.0, "fp32_tflops": 157.3}   # MI355X, dense
 PREFILL_TOKENS = 2048
 
+DESIGN_SIZES = {"360m": "smollm2-360m", "1.7b": "smollm2-1.7b", "8b": "llama-3-8b"}
+
+
+def sagalorn_like(shapes: dict, layers: int, window: int = 1024, keep_first: int = 64) -> dict:
+    """A Sagalorn configuration with the widths of a Llama one: the three mixers in turn, each layer with a feed-forward."""
+    d, H, G = shapes["hidden_size"], shapes["num_attention_heads"], shapes["num_key_value_heads"]
+    hd = shapes.get("head_dim") or d // H
+    mlp = {"kind": "dense", "ff": shapes["intermediate_size"]}
+    kinds = [
+        {"type": "retention", "mixer": {"heads": H, "dim": hd, "vdim": hd, "rot": {"dims": hd, "base": 10000.0},
+                                        "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, H - 1)) for h in range(H)]}, "mlp": mlp},
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                        "mask": {"size": window, "keep_first": keep_first}}, "mlp": mlp},
+        {"type": "gla", "mixer": {"heads": H, "dim": hd, "vdim": hd, "tau": 16.0, "rank": 64}, "mlp": mlp},
+    ]
+    return dict(architecture="Sagalorn", vocab=shapes["vocab_size"], width=d, streams=2, logit_scale=1.0,
+                embedding={"scale": 1.0}, norm={"eps": shapes["rms_norm_eps"]}, layers=[kinds[i % 3] for i in range(layers)])
+
+
+def design_bench(a) -> int:
+    """Prefill (one step of 2,048 tokens) and decode (batch and context as given, tokens fed back from the device sampler)
+    of a Sagalorn model and of the Llama of the same sizes, one after the other on the same GPU; one JSON line."""
+    import torch
+    from glassbox_amd.build import source_version
+    from glassbox_amd.config import config_from_dict
+    from glassbox_amd.engine import Engine
+    from glassbox_amd.sampling import greedy_pending
+    from glassbox_amd.weights import build_model, init_random
+
+    g = torch.Generator().manual_seed(1)
+    layers = a.layers or 12
+
+    def measure(raw: dict) -> dict:
+        cfg = config_from_dict(raw)
+        model = build_model(cfg)
+        init_random(model, seed=0, dtype=a.dtype, device="cuda:0")
+        vocab = model.vocab_size
+        eng = Engine(model, dtype=a.dtype, max_tokens=a.batch * (a.context + 64), max_seqs=a.batch, page_size=a.page_size,
+                     graph_decode=False if a.no_graph else None, layer_tapes=not a.no_layer_tapes)
+        times = []
+        for i in range(4):
+            toks = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step([(f"p{i}", toks, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            eng.end_request(f"p{i}")
+        out = {"prefill_tok_s": round(PREFILL_TOKENS / min(times[1:]), 1), "prefill_ms": round(min(times[1:]) * 1e3, 3)}
+        if a.only != "prefill":
+            names = [f"d{i}" for i in range(a.batch)]
+            start = a.context - a.steps - a.warmup
+            prompts = [torch.randint(0, vocab, (start,), generator=g).tolist() for _ in names]
+            for at in range(0, start - 1, PREFILL_TOKENS):
+                n = min(PREFILL_TOKENS, start - 1 - at)
+                for name, p in zip(names, prompts):
+                    eng.step([(name, p[at:at + n], [])])
+            tokens = [p[-1] for p in prompts]
+            for i in range(a.warmup + a.steps):
+                if i == a.warmup:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                tokens = greedy_pending(eng.step([(name, [t], [0]) for name, t in zip(names, tokens)]))
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / a.steps
+            out.update(decode_tok_s=round(a.batch / dt, 1), decode_ms=round(dt * 1e3, 4), graph=eng.decode_graphs is not None)
+            for name in names:
+                eng.end_request(name)
+        out["weight_gb"] = round(model.weight_bytes() / 1e9, 3)
+        del eng, model
+        torch.cuda.empty_cache()
+        return out
+
+    sizes = {}
+    for size in a.design_sizes.split(","):
+        shapes = SHAPES[DESIGN_SIZES[size]]
+        llama = dict(shapes, num_hidden_layers=layers, max_position_embeddings=max(shapes["max_position_embeddings"], a.context + 1))
+        sizes[size] = {"sagalorn": measure(sagalorn_like(shapes, layers)), "llama": measure(llama),
+                       "width": shapes["hidden_size"], "ff": shapes["intermediate_size"], "layers": layers}
+    print(json.dumps({"design": "Sagalorn", "beside": "LlamaForCausalLM", "dtype": a.dtype, "batch": a.batch, "context": a.context,
+                      "prefill_tokens": PREFILL_TOKENS, "steps": a.steps, "warmup": a.warmup, "sizes": sizes,
+                      "meta": {"gpu": torch.cuda.get_device_name(0), "commit": source_version(),
+                               "date": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ")}}))
+    return 0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -68,6 +159,9 @@ def main() -> int:
                     help="read a step's sampled tokens back before the next step is launched")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --only prefill, for profiling: a prompt of another length than the 2,048 tokens of the record")
+    ap.add_argument("--design", choices=["sagalorn"], default=None,
+                    help="instead of the record: models of this design at the sizes of --design-sizes beside Llamas of equal size")
+    ap.add_argument("--design-sizes", default="360m,1.7b", help="out of " + ", ".join(DESIGN_SIZES))
     a = ap.parse_args()
     if a.prefill_tokens != PREFILL_TOKENS and a.only != "prefill":
         print("bench.py: --prefill-tokens goes with --only prefill; the record's prefill is of 2,048 tokens")
@@ -75,6 +169,11 @@ def main() -> int:
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         return 2
+    if a.design is not None:
+        if any(s not in DESIGN_SIZES for s in a.design_sizes.split(",")):
+            print(f"bench.py: --design-sizes takes {', '.join(DESIGN_SIZES)}")
+            return 2
+        return design_bench(a)
 
     import torch
     from glassbox_amd.config import config_from_dict

@@ -600,16 +600,21 @@ extern "C" int gb_copy_rows(void* base, long long row_bytes, const int32_t* src,
 // For attention whose values are its keys as projected: row t of `qk` holds nh query heads, then nkv key heads.
 // x = projection + bias; a key head's x goes to the value pages as it is; then every head is RMS-normed over its
 // hd dimensions with a weight shared by the heads (w_q for queries, w_k for keys): queries are written back in
-// place, keys into the key pages.  One wave a (token, head); sums and the norm in 32-bit.
+// place, keys into the key pages.  With v_off >= 0 nothing goes to pages: the normed keys stay in place too and the
+// values are written to the same rows from column v_off on (a kernel that writes whole pages' worth of a step's rows
+// takes them from there).  One wave a (token, head), four a workgroup; sums and the norm in 32-bit.
 template <typename T>
-__global__ __launch_bounds__(kWave) void qk_norm_store_kernel(T* __restrict__ qk, int stride, const float* __restrict__ bias_q,
-                                                            const float* __restrict__ bias_k, const float* __restrict__ w_q,
-                                                            const float* __restrict__ w_k, float eps,
-                                                            const int32_t* __restrict__ slots, T* __restrict__ k_pages,
-                                                            T* __restrict__ v_pages, int nh, int nkv, int hd, int page_size) {
-  const int t = blockIdx.x / (nh + nkv), h = blockIdx.x % (nh + nkv);
+__global__ __launch_bounds__(4 * kWave) void qk_norm_store_kernel(T* __restrict__ qk, int stride, const float* __restrict__ bias_q,
+                                                                const float* __restrict__ bias_k, const float* __restrict__ w_q,
+                                                                const float* __restrict__ w_k, float eps,
+                                                                const int32_t* __restrict__ slots, T* __restrict__ k_pages,
+                                                                T* __restrict__ v_pages, int nh, int nkv, int hd, int page_size,
+                                                                int v_off, int pairs) {
+  const int pair = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (pair >= pairs) return;
+  const int t = pair / (nh + nkv), h = pair % (nh + nkv);
   const bool is_key = h >= nh;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x % kWave;
   T* row = qk + (size_t)t * stride + (size_t)h * hd;
   const float* bias = is_key ? (bias_k ? bias_k + (size_t)(h - nh) * hd : nullptr) : (bias_q ? bias_q + (size_t)h * hd : nullptr);
   const float* w = is_key ? w_k : w_q;
@@ -643,8 +648,9 @@ __global__ __launch_bounds__(kWave) void qk_norm_store_kernel(T* __restrict__ qk
     const int d = lane + j * kWave;
     if (d >= hd) continue;
     const float y = w ? w[d] * (x[j] * s) : x[j];
-    if (!is_key) {
+    if (!is_key || v_off >= 0) {
       row[d] = from_f<T>(y);
+      if (is_key) qk[(size_t)t * stride + v_off + (size_t)(h - nh) * hd + d] = from_f<T>(x[j]);
     } else if (slot >= 0) {
       kb[key_offset(slot % page_size, d, page_size, piece)] = from_f<T>(y);
       vb[(size_t)d * page_size + slot % page_size] = from_f<T>(x[j]);
@@ -654,20 +660,23 @@ __global__ __launch_bounds__(kWave) void qk_norm_store_kernel(T* __restrict__ qk
 
 extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bias_q, const float* bias_k, const float* w_q,
                                 const float* w_k, float eps, const int32_t* slots, void* k_pages, void* v_pages, int n,
-                                int nh, int nkv, int hd, int page_size, hipStream_t stream) {
+                                int nh, int nkv, int hd, int page_size, int v_off, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && hd > 0 && hd <= 4 * kWave, "qk_norm_store: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh,
              nkv, hd);
   GB_REQUIRE(stride >= (nh + nkv) * hd, "qk_norm_store: rows of %d hold fewer than %d heads of %d", stride, nh + nkv, hd);
   GB_REQUIRE(slots == nullptr || (k_pages && v_pages && page_size > 0), "qk_norm_store: cache rows without pages");
+  GB_REQUIRE(v_off < 0 || (slots == nullptr && v_off >= (nh + nkv) * hd && v_off + nkv * hd <= stride),
+             "qk_norm_store: values in the rows lie behind the heads, and nothing goes to pages then");
   GB_REQUIRE((long long)n * (nh + nkv) < (1ll << 31), "qk_norm_store: too many (token, head) pairs");
   if (n == 0) return 0;
-  const dim3 grid((unsigned)(n * (nh + nkv)));
+  const int pairs = n * (nh + nkv);
+  const dim3 grid((unsigned)((pairs + 3) / 4));
   if (dtype == kF32)
-    hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, dim3(kWave), 0, stream, (float*)qk, stride, bias_q, bias_k, w_q, w_k,
-                       eps, slots, (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size);
+    hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, dim3(4 * kWave), 0, stream, (float*)qk, stride, bias_q, bias_k, w_q, w_k,
+                       eps, slots, (float*)k_pages, (float*)v_pages, nh, nkv, hd, page_size, v_off, pairs);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, dim3(kWave), 0, stream, (bf16*)qk, stride, bias_q, bias_k, w_q, w_k, eps,
-                       slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size);
+    hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, dim3(4 * kWave), 0, stream, (bf16*)qk, stride, bias_q, bias_k, w_q, w_k,
+                       eps, slots, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, page_size, v_off, pairs);
   else
     return fail("qk_norm_store: unknown dtype %d", dtype);
   return launched("qk_norm_store");

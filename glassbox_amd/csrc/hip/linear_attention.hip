@@ -12,6 +12,14 @@
 // q, k and decays through LDS sixteen tokens at a time, the next sixteen on their way from memory meanwhile.
 // q, k and the decays come in 32-bit (what the kernels below prepare), v in the activations' type.
 //
+// A long portion of a prompt would leave the chip to the few waves of its request, one token after the other.  It is
+// cut into segments of `seg_len` tokens that run side by side: segment 0 goes on from the request's state, every other
+// one starts from nothing and leaves its own end state E and the product D of its decays in a workspace.  A second
+// kernel gives a segment the state S0 it should have started from (folded from the segments before it:
+// S <- D S + E) and adds what that state contributes to each token's output, (q_t * P_t)^T S0 with P_t the product of
+// the decays from the segment's first token to t; the last segment writes the request's state, D S0 + E.  Portions of
+// up to `seg_len` tokens take none of this.
+//
 // Around it: `retention_prep` (rotation of the first `rot` dimensions of the q and k heads in rotate-half pairs,
 // k scaled), `gla_prep` (q scaled, decays sigmoid(z)^(1/tau) from the low-rank projection z = A2 t + b), and
 // `head_norm_gate` (each head's output divided by its root mean square, an optional weight over dv, times
@@ -31,30 +39,61 @@ constexpr int kWaves = 4;
 constexpr int kColsBlock = kColsWave * kWaves;
 constexpr int kThreads = kWaves * kWave;
 
+// Sum over the eight lanes of a column (lanes 8c .. 8c+7), by data-parallel moves inside the wave's rows of 16 lanes:
+// neighbours, pairs of neighbours, then the other half of the eight.  Every lane of the eight gets the sum.
+__device__ __forceinline__ float sum8(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  return v;
+}
+
+// What a workgroup of either kernel works on: its request's segment.
+struct Segment {
+  int seq, seg, n_segs, first, count;
+  __device__ __forceinline__ Segment(const int32_t* q_start, const int32_t* q_len, int z, int segs, int seg_len) {
+    seq = z / segs;
+    seg = z % segs;
+    const int all = q_len[seq];
+    n_segs = segs > 1 ? (all + seg_len - 1) / seg_len : 1;
+    first = q_start[seq] + seg * seg_len;
+    count = n_segs > 1 ? min(seg_len, all - seg * seg_len) : all;
+  }
+};
+
 template <typename T, int R, bool GATED>
 __global__ __launch_bounds__(kThreads) void scan_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ a, const float* __restrict__ head_decay,
     const T* __restrict__ v, int v_stride, float* __restrict__ out, float* __restrict__ state,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
-    const int32_t* __restrict__ state_slots, int nh, int dk, int dv) {
+    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int segs, int seg_len, float* __restrict__ seg_state,
+    float* __restrict__ seg_decay) {
   constexpr int DKP = R * kLanesCol;                       // rows, padded
   constexpr int PER = (kTokens * DKP) / kThreads;          // staged elements a thread and array (R >= 2)
   __shared__ float qs[kTokens][DKP], ks[kTokens][DKP], ds[GATED ? kTokens : 1][GATED ? DKP : 1];
   __shared__ float vs[kTokens][kColsBlock];
-  const int seq = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kColsBlock;
+  const Segment sg(q_start, q_len, blockIdx.z, segs, seg_len);
+  if (sg.seg >= sg.n_segs) return;
+  const int seq = sg.seq, h = blockIdx.y, col0 = blockIdx.x * kColsBlock;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int rg = lane % kLanesCol;                          // which R rows of the column
   const int cb = wave * kColsWave + lane / kLanesCol;       // column within the block
   const int col = col0 + cb;
-  const int first = q_start[seq], count = q_len[seq];
+  const int first = sg.first, count = sg.count;
   const int width = nh * dk;
   const bool live = col < dv;
+  const bool cut = sg.n_segs > 1;                           // the request's portion runs as several segments
 
-  float S[R];
-  float* srow = state + (((size_t)state_slots[seq] * nh + h) * dv + (live ? col : 0)) * dk + rg * R;
-  const bool fresh = pos0[seq] == 0;   // a request's first tokens start from an empty state, whatever the slot held
+  float S[R], P[GATED ? R : 1];
+  float* slot_row = state + (((size_t)state_slots[seq] * nh + h) * dv + (live ? col : 0)) * dk + rg * R;
+  // where the end state goes: the request's slot, or, of a segment, the workspace
+  float* srow = cut ? seg_state + (((size_t)blockIdx.z * nh + h) * dv + (live ? col : 0)) * dk + rg * R : slot_row;
+  // a request's first tokens start from an empty state, whatever the slot held; so does every segment but the first
+  const bool fresh = pos0[seq] == 0 || sg.seg > 0;
 #pragma unroll
-  for (int m = 0; m < R; ++m) S[m] = (!fresh && live && rg * R + m < dk) ? srow[m] : 0.f;
+  for (int m = 0; m < R; ++m) S[m] = (!fresh && live && rg * R + m < dk) ? slot_row[m] : 0.f;
+#pragma unroll
+  for (int m = 0; m < (GATED ? R : 1); ++m) P[m] = 1.f;
   const float decay = GATED ? 1.f : head_decay[h];
 
   float nq[PER], nk[PER], na[GATED ? PER : 1], nv[2];
@@ -92,27 +131,151 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(
     __syncthreads();
     if (t0 + kTokens < count) fetch(t0 + kTokens);
     const int here = min(kTokens, count - t0);
-    for (int j = 0; j < here; ++j) {
+    // U tokens at a time: their operands are read from LDS together, the state goes through them in order (one
+    // multiply-add a token and row is all that waits for the token before), and their outputs' sums over the rows and
+    // over the eight lanes of a column run side by side
+    constexpr int U = R <= 8 ? 4 : R == 16 ? 2 : 1;
+    float* orow = out + (size_t)(first + t0) * ((size_t)nh * dv) + (size_t)h * dv + col;
+    int j = 0;
+    for (; j + U <= here; j += U) {
+      float kk[U][R], qq[U][R], aa[GATED ? U : 1][GATED ? R : 1], vv[U], part[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        vv[u] = vs[j + u][cb];
+#pragma unroll
+        for (int m = 0; m < R; ++m) {
+          kk[u][m] = ks[j + u][rg * R + m];
+          qq[u][m] = qs[j + u][rg * R + m];
+          if (GATED) aa[u][m] = ds[j + u][rg * R + m];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        part[u] = 0.f;
+#pragma unroll
+        for (int m = 0; m < R; ++m) {
+          S[m] = fmaf(GATED ? aa[u][m] : decay, S[m], kk[u][m] * vv[u]);
+          part[u] = fmaf(S[m], qq[u][m], part[u]);
+        }
+        if (GATED && cut) {
+#pragma unroll
+          for (int m = 0; m < R; ++m) P[m] *= aa[u][m];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) part[u] = sum8(part[u]);
+      if (rg == 0 && live) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) orow[(size_t)(j + u) * ((size_t)nh * dv)] = part[u];
+      }
+    }
+    for (; j < here; ++j) {   // the same sums, token by token
       const float vv = vs[j][cb];
       float part = 0.f;
 #pragma unroll
       for (int m = 0; m < R; ++m) {
-        const float kk = ks[j][rg * R + m], qq = qs[j][rg * R + m];
-        const float aa = GATED ? ds[j][rg * R + m] : decay;
-        S[m] = fmaf(aa, S[m], kk * vv);
-        part = fmaf(S[m], qq, part);
+        S[m] = fmaf(GATED ? ds[j][rg * R + m] : decay, S[m], ks[j][rg * R + m] * vv);
+        part = fmaf(S[m], qs[j][rg * R + m], part);
+        if (GATED && cut) P[m] *= ds[j][rg * R + m];
       }
-      // the eight lanes of a column, in a fixed order
-      part += __shfl_xor(part, 1, kWave);
-      part += __shfl_xor(part, 2, kWave);
-      part += __shfl_xor(part, 4, kWave);
-      if (rg == 0 && live) out[(size_t)(first + t0 + j) * ((size_t)nh * dv) + (size_t)h * dv + col] = part;
+      part = sum8(part);
+      if (rg == 0 && live) orow[(size_t)j * ((size_t)nh * dv)] = part;
     }
   }
   if (live) {
 #pragma unroll
     for (int m = 0; m < R; ++m)
       if (rg * R + m < dk) srow[m] = S[m];
+  }
+  if (GATED && cut && blockIdx.x == 0 && cb == 0) {   // the segment's decays, once a head
+    float* drow = seg_decay + ((size_t)blockIdx.z * nh + h) * dk + rg * R;
+#pragma unroll
+    for (int m = 0; m < R; ++m)
+      if (rg * R + m < dk) drow[m] = P[m];
+  }
+}
+
+// The second kernel of a portion that ran as segments (see the top of the file): same grid, same lanes.
+template <int R, bool GATED>
+__global__ __launch_bounds__(kThreads) void scan_join_kernel(
+    const float* __restrict__ q, const float* __restrict__ a, const float* __restrict__ head_decay, float* __restrict__ out,
+    float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int segs, int seg_len, const float* __restrict__ seg_state,
+    const float* __restrict__ seg_decay) {
+  constexpr int DKP = R * kLanesCol;
+  constexpr int PER = (kTokens * DKP) / kThreads;
+  __shared__ float qs[kTokens][DKP], ds[GATED ? kTokens : 1][GATED ? DKP : 1];
+  const Segment sg(q_start, q_len, blockIdx.z, segs, seg_len);
+  if (sg.n_segs <= 1 || sg.seg == 0 || sg.seg >= sg.n_segs) return;   // nothing was cut, or the segment started from the state
+  const int h = blockIdx.y, col0 = blockIdx.x * kColsBlock;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int rg = lane % kLanesCol, cb = wave * kColsWave + lane / kLanesCol, col = col0 + cb;
+  const int first = sg.first, count = sg.count, width = nh * dk;
+  const bool live = col < dv;
+  const float decay = GATED ? 1.f : head_decay[h];
+  float whole = 1.f;   // a full segment's decay, for a decay a head: the same products in the same order as token by token
+  if (!GATED)
+    for (int i = 0; i < seg_len; ++i) whole *= decay;
+
+  // the state this segment should have started from: the end states of the segments before it, folded in order
+  const size_t cell0 = (size_t)sg.seq * segs;
+  auto e_row = [&](int sgm) { return seg_state + ((((cell0 + sgm) * nh + h) * dv + (live ? col : 0)) * dk) + rg * R; };
+  float S0[R];
+#pragma unroll
+  for (int m = 0; m < R; ++m) S0[m] = (live && rg * R + m < dk) ? e_row(0)[m] : 0.f;
+  for (int sgm = 1; sgm < sg.seg; ++sgm) {
+    const float* e = e_row(sgm);
+    const float* d = seg_decay + ((cell0 + sgm) * nh + h) * dk + rg * R;
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+      const bool ok = live && rg * R + m < dk;
+      S0[m] = fmaf(GATED ? (ok ? d[m] : 0.f) : whole, S0[m], ok ? e[m] : 0.f);
+    }
+  }
+
+  float P[R];   // the decays from the segment's first token on
+#pragma unroll
+  for (int m = 0; m < R; ++m) P[m] = 1.f;
+  float nq[PER], na[GATED ? PER : 1];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int idx = tid + e * kThreads, tok = idx / DKP, ch = idx % DKP;
+      const bool ok = t0 + tok < count && ch < dk;
+      const size_t at = (size_t)(first + t0 + tok) * width + (size_t)h * dk + ch;
+      nq[e] = ok ? q[at] : 0.f;
+      if (GATED) na[e] = ok ? a[at] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < count; t0 += kTokens) {
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      (&qs[0][0])[tid + e * kThreads] = nq[e];
+      if (GATED) (&ds[0][0])[tid + e * kThreads] = na[e];
+    }
+    __syncthreads();
+    if (t0 + kTokens < count) fetch(t0 + kTokens);
+    const int here = min(kTokens, count - t0);
+    float* orow = out + (size_t)(first + t0) * ((size_t)nh * dv) + (size_t)h * dv + col;
+    for (int j = 0; j < here; ++j) {
+      float part = 0.f;
+#pragma unroll
+      for (int m = 0; m < R; ++m) {
+        P[m] *= GATED ? ds[j][rg * R + m] : decay;
+        part = fmaf(qs[j][rg * R + m] * P[m], S0[m], part);
+      }
+      part = sum8(part);
+      if (rg == 0 && live) orow[(size_t)j * ((size_t)nh * dv)] += part;
+    }
+  }
+  if (sg.seg == sg.n_segs - 1 && live) {   // the request's state after the portion
+    const float* e = e_row(sg.seg);
+    float* srow = state + (((size_t)state_slots[sg.seq] * nh + h) * dv + col) * dk + rg * R;
+#pragma unroll
+    for (int m = 0; m < R; ++m)
+      if (rg * R + m < dk) srow[m] = fmaf(P[m], S0[m], e[m]);
   }
 }
 
@@ -147,34 +310,45 @@ __device__ __forceinline__ float log_sigmoid(float z) {
   return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
 }
 
-// q32 = q * q_scale, k32 = k, decay[t, c] = sigmoid(z)^(1/tau) with z = sum_r A2[c, r] low[t, r] + b[c]
+// q32 = q * q_scale, k32 = k, decay[t, c] = sigmoid(z)^(1/tau) with z = sum_r A2[c, r] low[t, r] + b[c]; with `zin`
+// the sums come from there (a matrix product made them) and a2 is not read
 template <typename T>
 __global__ void gla_prep_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int low_off,
-                                const T* __restrict__ a2, const float* __restrict__ a2_bias, float* __restrict__ q32,
+                                const T* __restrict__ a2, const float* __restrict__ zin,
+                                const float* __restrict__ a2_bias, float* __restrict__ q32,
                                 float* __restrict__ k32, float* __restrict__ decay, int width, int rank, float q_scale,
                                 float inv_tau) {
   extern __shared__ float low[];   // [rank]
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * stride;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = to_f(row[low_off + r]);
-  __syncthreads();
+  if (!zin) {
+    for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = to_f(row[low_off + r]);
+    __syncthreads();
+  }
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     q32[(size_t)t * width + c] = to_f(row[q_off + c]) * q_scale;
     k32[(size_t)t * width + c] = to_f(row[k_off + c]);
     float z = 0.f;
-    const T* w = a2 + (size_t)c * rank;
-    for (int r = 0; r < rank; ++r) z = fmaf(to_f(w[r]), low[r], z);
+    if (zin) {
+      z = zin[(size_t)t * width + c];
+    } else {
+      const T* w = a2 + (size_t)c * rank;
+      for (int r = 0; r < rank; ++r) z = fmaf(to_f(w[r]), low[r], z);
+    }
     z += a2_bias ? a2_bias[c] : 0.f;
     decay[(size_t)t * width + c] = expf(log_sigmoid(z) * inv_tau);
   }
 }
 
-// out[t, h, :] = w * o / sqrt(mean(o^2) + eps) * silu(gate[t, h, :])  (w == nullptr: no weight).  One wave a (token, head).
+// out[t, h, :] = w * o / sqrt(mean(o^2) + eps) * silu(gate[t, h, :])  (w == nullptr: no weight).  One wave a (token, head),
+// four waves a workgroup.
 template <typename T>
-__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
-                                                             int gate_stride, const float* __restrict__ w,
-                                                             T* __restrict__ out, int nh, int dv, float eps) {
-  const int t = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
+__global__ __launch_bounds__(4 * kWave) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                                 int gate_stride, const float* __restrict__ w,
+                                                                 T* __restrict__ out, int nh, int dv, float eps, int pairs) {
+  const int pair = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (pair >= pairs) return;
+  const int t = pair / nh, h = pair % nh, lane = threadIdx.x % kWave;
   const float* orow = o + ((size_t)t * nh + h) * dv;
   float ss = 0.f;
   for (int d = lane; d < dv; d += kWave) ss = fmaf(orow[d], orow[d], ss);
@@ -191,11 +365,15 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(const float* __re
 template <typename T, bool GATED>
 int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const float* k, const float* a, const float* head_decay,
                 const void* v, int v_stride, float* out, float* state, const int32_t* q_start, const int32_t* q_len,
-                const int32_t* pos0, const int32_t* slots, int nh, int dk, int dv) {
+                const int32_t* pos0, const int32_t* slots, int nh, int dk, int dv, int segs, int seg_len, float* seg_state,
+                float* seg_decay) {
 #define GB_SCAN(RR)                                                                                                          \
   case RR:                                                                                                                   \
     hipLaunchKernelGGL((scan_kernel<T, RR, GATED>), grid, dim3(kThreads), 0, stream, q, k, a, head_decay, (const T*)v, v_stride, \
-                       out, state, q_start, q_len, pos0, slots, nh, dk, dv);                                                 \
+                       out, state, q_start, q_len, pos0, slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);            \
+    if (segs > 1)                                                                                                            \
+      hipLaunchKernelGGL((scan_join_kernel<RR, GATED>), grid, dim3(kThreads), 0, stream, q, a, head_decay, out, state, q_start, \
+                         q_len, slots, nh, dk, dv, segs, seg_len, (const float*)seg_state, (const float*)seg_decay);         \
     break;
   switch (R) {
     GB_SCAN(2) GB_SCAN(4) GB_SCAN(8) GB_SCAN(16) GB_SCAN(32)
@@ -211,26 +389,39 @@ int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const floa
 // nullptr with head_decay [nh] float32; v rows of nh * dv in the activations' type (row stride v_stride); out [n, nh * dv]
 // float32; state [slots, nh, dv, dk] float32.  Request s of the step brings rows q_start[s] .. + q_len[s] - 1, starts at
 // position pos0[s] (0: from an empty state) and keeps its state in slot state_slots[s].
+// segs > 1: no request brings more than segs * seg_len rows, and those that bring more than seg_len run as segments of
+// seg_len rows side by side; seg_ws holds gb_linear_scan_floats(n_seqs, nh, dk, dv, segs) floats.
+extern "C" long long gb_linear_scan_floats(int n_seqs, int nh, int dk, int dv, int segs) {
+  return segs > 1 ? (long long)n_seqs * segs * nh * ((long long)dv * dk + dk) : 0;
+}
+
 extern "C" int gb_linear_scan(const float* q, const float* k, const float* a, const float* head_decay, const void* v,
                               int v_dtype, int v_stride, float* out, float* state, const int32_t* q_start,
                               const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
-                              int dk, int dv, hipStream_t stream) {
+                              int dk, int dv, int segs, int seg_len, float* seg_ws, long long seg_ws_floats,
+                              hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes requests=%d heads=%d dk=%d dv=%d", n_seqs, nh, dk, dv);
   GB_REQUIRE(dk <= 32 * kLanesCol, "linear_scan: a key size of %d is above the supported %d", dk, 32 * kLanesCol);
   GB_REQUIRE((a != nullptr) != (head_decay != nullptr), "linear_scan: a decay a head or a decay a key channel, one of the two");
   GB_REQUIRE(v_stride >= nh * dv, "linear_scan: value rows of %d hold fewer than %d heads of %d", v_stride, nh, dv);
-  GB_REQUIRE(n_seqs <= 65535 && nh <= 65535, "linear_scan: too many requests or heads for one launch");
+  GB_REQUIRE(segs >= 1 && (segs == 1 || (seg_len >= kTokens && seg_ws != nullptr &&
+                                          seg_ws_floats >= gb_linear_scan_floats(n_seqs, nh, dk, dv, segs))),
+             "linear_scan: %d segments of %d rows need a workspace of %lld floats", segs, seg_len,
+             gb_linear_scan_floats(n_seqs, nh, dk, dv, segs));
+  GB_REQUIRE((long long)n_seqs * segs <= 65535 && nh <= 65535, "linear_scan: too many requests, segments or heads for one launch");
   if (n_seqs == 0) return 0;
+  float* seg_state = seg_ws;
+  float* seg_decay = segs > 1 ? seg_ws + (size_t)n_seqs * segs * nh * dv * dk : nullptr;
   int R = 2;
   while (R * kLanesCol < dk) R *= 2;
-  const dim3 grid((unsigned)((dv + kColsBlock - 1) / kColsBlock), (unsigned)nh, (unsigned)n_seqs);
+  const dim3 grid((unsigned)((dv + kColsBlock - 1) / kColsBlock), (unsigned)nh, (unsigned)(n_seqs * segs));
   const bool gated = a != nullptr;
   if (v_dtype == kF32)
-    return gated ? launch_scan<float, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv)
-                 : launch_scan<float, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv);
+    return gated ? launch_scan<float, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay)
+                 : launch_scan<float, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);
   if (v_dtype == kBF16)
-    return gated ? launch_scan<bf16, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv)
-                 : launch_scan<bf16, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv);
+    return gated ? launch_scan<bf16, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay)
+                 : launch_scan<bf16, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);
   return fail("linear_scan: unknown dtype %d", v_dtype);
 }
 
@@ -255,9 +446,10 @@ extern "C" int gb_retention_prep(const void* proj, int dtype, int stride, int q_
 }
 
 extern "C" int gb_gla_prep(const void* proj, int dtype, int stride, int q_off, int k_off, int low_off, const void* a2,
-                           const float* a2_bias, float* q32, float* k32, float* decay, int n, int width, int rank,
+                           const float* zin, const float* a2_bias, float* q32, float* k32, float* decay, int n, int width, int rank,
                            float q_scale, float inv_tau, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && width > 0 && rank > 0 && rank <= 4096, "gla_prep: bad sizes n=%d width=%d rank=%d", n, width, rank);
+  GB_REQUIRE(a2 != nullptr || zin != nullptr, "gla_prep: neither the decay's second matrix nor its products");
   GB_REQUIRE(q_off >= 0 && k_off >= 0 && low_off >= 0 && q_off + width <= stride && k_off + width <= stride &&
                  low_off + rank <= stride, "gla_prep: heads beyond the row");
   if (n == 0) return 0;
@@ -265,10 +457,10 @@ extern "C" int gb_gla_prep(const void* proj, int dtype, int stride, int q_off, i
   const size_t smem = sizeof(float) * rank;
   if (dtype == kF32)
     hipLaunchKernelGGL(gla_prep_kernel<float>, dim3(n), dim3(threads), smem, stream, (const float*)proj, stride, q_off, k_off,
-                       low_off, (const float*)a2, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
+                       low_off, (const float*)a2, zin, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(gla_prep_kernel<bf16>, dim3(n), dim3(threads), smem, stream, (const bf16*)proj, stride, q_off, k_off,
-                       low_off, (const bf16*)a2, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
+                       low_off, (const bf16*)a2, zin, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
   else
     return fail("gla_prep: unknown dtype %d", dtype);
   return launched("gla_prep");
@@ -280,11 +472,11 @@ extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, in
   GB_REQUIRE((long long)n * nh < (1ll << 31), "head_norm_gate: too many (token, head) pairs");
   if (n == 0) return 0;
   if (dtype == kF32)
-    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3((unsigned)(n * nh)), dim3(kWave), 0, stream, o, (const float*)gate,
-                       gate_stride, w, (float*)out, nh, dv, eps);
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3((unsigned)((n * nh + 3) / 4)), dim3(4 * kWave), 0, stream, o,
+                       (const float*)gate, gate_stride, w, (float*)out, nh, dv, eps, n * nh);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(head_norm_gate_kernel<bf16>, dim3((unsigned)(n * nh)), dim3(kWave), 0, stream, o, (const bf16*)gate,
-                       gate_stride, w, (bf16*)out, nh, dv, eps);
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16>, dim3((unsigned)((n * nh + 3) / 4)), dim3(4 * kWave), 0, stream, o,
+                       (const bf16*)gate, gate_stride, w, (bf16*)out, nh, dv, eps, n * nh);
   else
     return fail("head_norm_gate: unknown dtype %d", dtype);
   return launched("head_norm_gate");

@@ -48,8 +48,8 @@ _SIGS = {
         "gb_rope_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _vp],
         "gb_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
         "gb_copy_rows": [_vp, C.c_longlong, _vp, _vp, _i, _vp],
-        # qk, dtype, stride, bias_q, bias_k, w_q, w_k, eps, slots, k, v, n, nh, nkv, hd, page, stream
-        "gb_qk_norm_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+        # qk, dtype, stride, bias_q, bias_k, w_q, w_k, eps, slots, k, v, n, nh, nkv, hd, page, v_off, stream
+        "gb_qk_norm_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
         "gb_add_bias": [_vp, _vp, _i, _i, _vp],
         "gb_scale_rows": [_vp, _f, C.c_longlong, _vp],
     },
@@ -60,12 +60,13 @@ _SIGS = {
     },
     "linear_attention": {
         # q, k, decays, head decays, v, v dtype, v stride, out, state, q_start, q_len, pos0, state slots, requests, heads,
-        # dk, dv, stream
-        "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+        # dk, dv, segments, rows a segment, workspace, its floats, stream
+        "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp,
+                           C.c_longlong, _vp],
         # proj, dtype, stride, q_off, k_off, cos, sin, q32, k32, n, heads, dk, rot, k_scale, stream
         "gb_retention_prep": [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
-        # proj, dtype, stride, q_off, k_off, low_off, a2, a2 bias, q32, k32, decay, n, width, rank, q_scale, 1/tau, stream
-        "gb_gla_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _vp],
+        # proj, dtype, stride, q_off, k_off, low_off, a2, z, a2 bias, q32, k32, decay, n, width, rank, q_scale, 1/tau, stream
+        "gb_gla_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _vp],
         # o, gate, dtype, gate stride, w, out, n, heads, dv, eps, stream
         "gb_head_norm_gate": [_vp, _vp, _i, _i, _vp, _vp, _i, _i, _i, _f, _vp],
     },
@@ -470,11 +471,13 @@ def copy_rows(base: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
 def qk_norm_store(qk: torch.Tensor, bias_q: Optional[torch.Tensor], bias_k: Optional[torch.Tensor],
                   w_q: Optional[torch.Tensor], w_k: Optional[torch.Tensor], eps: float, slots: Optional[torch.Tensor],
                   k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv_heads: int,
-                  head_dim: int) -> None:
+                  head_dim: int, values_in_rows: bool = False) -> None:
     """Rows of query heads then key heads: adds the biases, writes each key head as it then is to the value pages
     (the values of such a layer are its keys as projected), RMS-norms every head over its dimensions with the weight
     that the heads of its kind share (None: the head stays as it is), and leaves queries in place and keys in the key
-    pages at ``slots`` (None: nothing is stored).  Biases and weights are float32."""
+    pages at ``slots`` (None: nothing is stored).  Biases and weights are float32.  ``values_in_rows`` (without
+    ``slots``): the rows have room for the value heads behind the key heads; the normed keys stay in place, the values
+    are written behind them, and ``rope_store`` without rotation takes both to the pages."""
     _dev(qk, bias_q, bias_k, w_q, w_k, slots, k_pages, v_pages)
     n = qk.shape[0]
     stride = _rows(qk, "qk")
@@ -482,8 +485,8 @@ def qk_norm_store(qk: torch.Tensor, bias_q: Optional[torch.Tensor], bias_k: Opti
                           (w_q, head_dim, "w_q"), (w_k, head_dim, "w_k")):
         if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != size):
             raise KernelError(f"qk_norm_store: {what} must be contiguous float32 of {size} entries")
-    if qk.shape[1] < (n_heads + n_kv_heads) * head_dim:
-        raise KernelError("qk_norm_store: rows shorter than the heads")
+    if qk.shape[1] < (n_heads + (2 if values_in_rows else 1) * n_kv_heads) * head_dim or (values_in_rows and slots is not None):
+        raise KernelError("qk_norm_store: rows shorter than the heads, or values in the rows together with cache rows")
     page_size = 0
     if slots is not None:
         _i32(slots, "slots", n)
@@ -492,7 +495,8 @@ def qk_norm_store(qk: torch.Tensor, bias_q: Optional[torch.Tensor], bias_k: Opti
             raise KernelError("qk_norm_store: pages do not have this layer's kv heads and head size")
     lib = _lib("elementwise")
     _launch(lib, lib.gb_qk_norm_store, _p(qk), dtype_code(qk), stride, _p(bias_q), _p(bias_k), _p(w_q), _p(w_k), float(eps),
-            _p(slots), _p(k_pages), _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size, _stream())
+            _p(slots), _p(k_pages), _p(v_pages), n, n_heads, n_kv_heads, head_dim, page_size,
+            (n_heads + n_kv_heads) * head_dim if values_in_rows else -1, _stream())
 
 
 def add_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
@@ -590,11 +594,14 @@ def retention_prep(proj: torch.Tensor, q_off: int, k_off: int, cos: Optional[tor
 
 
 def gla_prep(proj: torch.Tensor, q_off: int, k_off: int, low_off: int, a2: torch.Tensor, a2_bias: Optional[torch.Tensor],
-             q32: torch.Tensor, k32: torch.Tensor, decay: torch.Tensor, q_scale: float, tau: float) -> None:
+             q32: torch.Tensor, k32: torch.Tensor, decay: torch.Tensor, q_scale: float, tau: float,
+             z: Optional[torch.Tensor] = None) -> None:
     """q32 = q * q_scale, k32 = k, decay = sigmoid(z)^(1/tau) with z = a2 . low + a2_bias, all float32 [n, width], from
     the projection's rows (queries, keys and the low-rank rows at the given columns; ``a2`` [width, rank] in the
-    projection's type)."""
-    _dev(proj, a2, a2_bias, q32, k32, decay)
+    projection's type).  ``z`` (float32 [n, width]): the products a2 . low, where a matrix product has made them."""
+    _dev(proj, a2, a2_bias, q32, k32, decay, z)
+    if z is not None:
+        _f32_rows(z, (proj.shape[0], a2.shape[0]), "z")
     n = proj.shape[0]
     stride = _rows(proj, "proj")
     width, rank = a2.shape
@@ -607,18 +614,31 @@ def gla_prep(proj: torch.Tensor, q_off: int, k_off: int, low_off: int, a2: torch
     if max(q_off, k_off) + width > proj.shape[1] or low_off + rank > proj.shape[1]:
         raise KernelError("gla_prep: the heads lie beyond the projection's rows")
     lib = _lib("linear_attention")
-    _launch(lib, lib.gb_gla_prep, _p(proj), dtype_code(proj), stride, int(q_off), int(k_off), int(low_off), _p(a2),
+    _launch(lib, lib.gb_gla_prep, _p(proj), dtype_code(proj), stride, int(q_off), int(k_off), int(low_off), _p(a2), _p(z),
             _p(a2_bias), _p(q32), _p(k32), _p(decay), n, width, rank, float(q_scale), 1.0 / float(tau), _stream())
+
+
+LINEAR_SEGMENT = 128          # rows of a segment of a long portion
+LINEAR_SEGMENT_FROM = 256     # portions up to here run token after token from the request's state: no bit depends on the cut
+
+
+def linear_scan_segments(max_q_len: int) -> int:
+    """Into how many segments ``linear_scan`` cuts the portions of a step whose longest one has ``max_q_len`` rows."""
+    return 1 if max_q_len <= LINEAR_SEGMENT_FROM else -(-max_q_len // LINEAR_SEGMENT)
 
 
 def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torch.Tensor, state: torch.Tensor, ctx,
                 n_heads: int, key_dim: int, value_dim: int, decay: Optional[torch.Tensor] = None,
-                head_decay: Optional[torch.Tensor] = None) -> None:
+                head_decay: Optional[torch.Tensor] = None, segments: int = 1,
+                workspace: Optional[torch.Tensor] = None) -> None:
     """The recurrence S <- diag(a) S + k v^T, o = S^T q over each request's rows of the step, in their order, from the
     state in the request's slot (empty for a request at position 0) and back into it.  ``decay`` float32
     [n, heads * key_dim] (a decay a key channel and token) or ``head_decay`` float32 [heads]; ``v`` rows of
     heads * value_dim in the activations' type (may be a view into wider rows); ``out`` float32 [n, heads * value_dim];
-    ``state`` float32 [slots, heads, value_dim, key_dim]."""
+    ``state`` float32 [slots, heads, value_dim, key_dim].  ``segments`` > 1 (``linear_scan_segments`` of the step's
+    longest portion, with a float32 ``workspace`` of requests * segments * heads * (value_dim + 1) * key_dim elements): long
+    portions run as segments of ``LINEAR_SEGMENT`` rows side by side and a second kernel joins them; what a token gets then
+    differs from the token-by-token sums by rounding."""
     _dev(q32, k32, v, out, state, decay, head_decay)
     n = q32.shape[0]
     _f32_rows(q32, (n, n_heads * key_dim), "q32")
@@ -636,10 +656,16 @@ def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torc
         raise KernelError("linear_scan: state must be contiguous float32 [slots, heads, value_dim, key_dim]")
     if key_dim > LINEAR_MAX_KEY_DIM:
         raise KernelError(f"linear_scan: a key size of {key_dim} is above {LINEAR_MAX_KEY_DIM}")
+    if segments > 1:
+        _dev(workspace)
+        need = ctx.num_seqs * segments * n_heads * (value_dim + 1) * key_dim
+        if workspace is None or workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() < need:
+            raise KernelError(f"linear_scan: {segments} segments need a contiguous float32 workspace of {need} elements")
     lib = _lib("linear_attention")
     _launch(lib, lib.gb_linear_scan, _p(q32), _p(k32), _p(decay), _p(head_decay), _p(v), dtype_code(v), _rows(v, "v"), _p(out),
             _p(state), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0), _p(ctx.state_slots), ctx.num_seqs, n_heads, key_dim,
-            value_dim, _stream())
+            value_dim, int(segments), LINEAR_SEGMENT, _p(workspace) if segments > 1 else None,
+            workspace.numel() if segments > 1 else 0, _stream())
 
 
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor, n_heads: int,

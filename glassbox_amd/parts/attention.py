@@ -211,12 +211,23 @@ class TiedValueAttention(Mixer):
         if cache is None or cache.k_pages is None:
             raise ValueError("TiedValueAttention needs a layer cache with pages")
         n = h.shape[0]
-        qk = ctx.buffer("qk", (n, self.q_dim + self.kv_dim), ctx.dtype)
-        ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
         slots = ctx.slots[cache.group] if cache.writable else None
-        ops.qk_norm_store(qk, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, slots,
-                          cache.k_pages if slots is not None else None, cache.v_pages if slots is not None else None,
-                          self.n_heads, self.n_kv_heads, self.head_dim)
+        if n > ops.ROPE_PRODUCT_MAX_ROWS and slots is not None:
+            # many rows: values are written into the rows behind the keys, and the kernel that takes a step's keys and
+            # values to their pages in whole lines does the cache write (no rotation)
+            rows = ctx.buffer("qkv", (n, self.q_dim + 2 * self.kv_dim), ctx.dtype)
+            qk = rows[:, :self.q_dim + self.kv_dim]
+            ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
+            ops.qk_norm_store(rows, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, None, None, None,
+                              self.n_heads, self.n_kv_heads, self.head_dim, values_in_rows=True)
+            ops.rope_store(rows, None, None, slots, cache.k_pages, cache.v_pages, self.n_heads, self.n_kv_heads,
+                           self.head_dim, rotate=False, portions=ctx.portions())
+        else:
+            qk = ctx.buffer("qk", (n, self.q_dim + self.kv_dim), ctx.dtype)
+            ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
+            ops.qk_norm_store(qk, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, slots,
+                              cache.k_pages if slots is not None else None, cache.v_pages if slots is not None else None,
+                              self.n_heads, self.n_kv_heads, self.head_dim)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         paged_attention(ctx, qk[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window, self.keep_first)
         ops.gemm(att, self.wo, residual, accumulate=not store, workspace=split_workspace(ctx, n, self.width, self.q_dim))

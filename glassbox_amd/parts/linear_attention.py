@@ -55,6 +55,15 @@ class _LinearMixer(Mixer):
                                f"kernel takes"))
         return out
 
+    @staticmethod
+    def _stack(parts):
+        """The rows of several matrices as one, filled up with rows of zeros to a multiple of 8 (rows of the product's
+        result then begin at 16-byte words whatever the sizes)."""
+        rows = sum(p.shape[0] for p in parts)
+        if rows % 8:
+            parts = list(parts) + [torch.zeros((8 - rows % 8, parts[0].shape[1]), dtype=parts[0].dtype, device=parts[0].device)]
+        return torch.cat(parts, 0)
+
     def _project(self, ctx, h):
         n = h.shape[0]
         proj = ctx.buffer("lin_proj", (n, self.w_in.shape[0]), ctx.dtype)
@@ -67,8 +76,14 @@ class _LinearMixer(Mixer):
             raise ValueError(f"{type(self).__name__} needs a layer cache with state")
         v_off, g_off = 2 * self.qk_dim, 2 * self.qk_dim + self.v_dim
         o = ctx.buffer("lin_o", (n, self.v_dim), torch.float32)
+        # a long portion runs as segments side by side (the step's longest portion decides for the whole launch)
+        segments = ops.linear_scan_segments(int(ctx.host["max_q_len"]))
+        ws = None
+        if segments > 1:
+            ws = ctx.buffer("lin_segments", (ctx.num_seqs * segments * self.n_heads * (self.value_dim + 1) * self.key_dim,),
+                            torch.float32)
         ops.linear_scan(q32, k32, proj[:, v_off:v_off + self.v_dim], o, cache.state, ctx, self.n_heads, self.key_dim,
-                        self.value_dim, decay=decay, head_decay=head_decay)
+                        self.value_dim, decay=decay, head_decay=head_decay, segments=segments, workspace=ws)
         gated = ctx.buffer("lin_gated", (n, self.v_dim), ctx.dtype)
         ops.head_norm_gate(o, proj[:, g_off:g_off + self.v_dim], norm_weight, gated, self.n_heads, self.value_dim, self.eps)
         ops.gemm(gated, self.wo, residual, accumulate=not store,
@@ -94,7 +109,7 @@ class Retention(_LinearMixer):
                 "o": TensorSpec((self.width, self.v_dim))}
 
     def load(self, tensors):
-        self.w_in = torch.cat([tensors[n] for n in ("q", "k", "v", "g")], 0)   # one product computes all four
+        self.w_in = self._stack([tensors[n] for n in ("q", "k", "v", "g")])   # one product computes all four
         self.wo = tensors["o"].contiguous()
         self.head_decay = torch.tensor(self.decay, dtype=torch.float32, device=self.wo.device)
 
@@ -136,7 +151,7 @@ class GatedLinearAttention(_LinearMixer):
         if tensors["a1"].shape[0] != tensors["a2"].shape[1]:
             raise ValueError(f"a1 has {tensors['a1'].shape[0]} rows, a2 has {tensors['a2'].shape[1]} columns")
         # one product computes q, k, v, the gate and the narrow rows of the decay
-        self.w_in = torch.cat([tensors[n] for n in ("q", "k", "v", "g", "a1")], 0)
+        self.w_in = self._stack([tensors[n] for n in ("q", "k", "v", "g", "a1")])
         self.wo = tensors["o"].contiguous()
         self.w_a2 = tensors["a2"].contiguous()
         self.a2_bias = tensors["a2.b"].contiguous()
@@ -152,6 +167,12 @@ class GatedLinearAttention(_LinearMixer):
         q32 = ctx.buffer("lin_q", (n, self.qk_dim), torch.float32)
         k32 = ctx.buffer("lin_k", (n, self.qk_dim), torch.float32)
         decay = ctx.buffer("lin_decay", (n, self.qk_dim), torch.float32)
-        ops.gla_prep(proj, 0, self.qk_dim, 2 * self.qk_dim + 2 * self.v_dim, self.w_a2, self.a2_bias, q32, k32, decay,
-                     1.0 / math.sqrt(self.key_dim), self.tau)
+        low_off, rank = 2 * self.qk_dim + 2 * self.v_dim, self.w_a2.shape[1]
+        z = None
+        if n > ops.FUSED_NORM_MAX_ROWS and (ctx.dtype == torch.float32 or (rank % 8 == 0 and low_off % 8 == 0)):
+            # many rows: the second matrix of the decay's projection as a product of its own (few rows: inside the kernel)
+            z = ctx.buffer("lin_z", (n, self.qk_dim), torch.float32)
+            ops.gemm(proj[:, low_off:low_off + rank], self.w_a2, z)
+        ops.gla_prep(proj, 0, self.qk_dim, low_off, self.w_a2, self.a2_bias, q32, k32, decay,
+                     1.0 / math.sqrt(self.key_dim), self.tau, z=z)
         self._finish(ctx, proj, q32, k32, residual, cache, store, self.norm_weight, decay=decay)

@@ -74,6 +74,48 @@ def test_the_recurrence_in_portions_of_a_batch(H, dk, dv, gated, vtype):
     assert torch.all(state[1] == 123.0) and torch.all(state[4] == 123.0)   # nobody else's slot was touched
 
 
+@pytest.mark.parametrize("H, dk, dv, gated", [(2, 64, 64, False), (3, 24, 40, True), (1, 128, 16, True), (2, 16, 70, False)])
+def test_long_portions_run_as_segments(H, dk, dv, gated):
+    """Portions beyond 256 rows are cut into segments that run side by side and are joined by a second kernel: three
+    requests (one goes on from a state, one is too short to be cut, one brings a single token and then a long portion)
+    against the plain recurrence, and the states they leave by going on token after token."""
+    from glassbox_amd import ops
+    torch.manual_seed(dk * dv)
+    lens = [700, 130, 301]
+    cuts = [(400, 299, 1), (130, 0, 0), (1, 299, 1)]
+    slots = [1, 3, 0]
+    state = torch.full((4, H, dv, dk), -7.0, device=DEV)
+    data = []
+    for T in lens:
+        q, k = torch.randn(T, H, dk, dtype=F64), torch.randn(T, H, dk, dtype=F64) / math.sqrt(dk)
+        v = torch.randn(T, H, dv, dtype=F64)
+        decay = torch.rand(T, H, dk, dtype=F64) * 0.1 + 0.9 if gated else (torch.linspace(0.95, 0.999, H, dtype=F64)
+                                                                          .view(1, H, 1).expand(T, H, dk))
+        q, k, v, decay = (t.float().to(F64) for t in (q, k, v, decay))
+        data.append((q, k, v, decay, ps.decayed_state_outputs(q, k, v, decay)))
+    done = [0, 0, 0]
+    for step in range(3):
+        rows = [(s, done[s], done[s] + cuts[s][step]) for s in range(3) if cuts[s][step]]
+        cat = lambda i: torch.cat([data[s][i][a:b] for s, a, b in rows], 0)
+        n = sum(b - a for _, a, b in rows)
+        starts = np.cumsum([0] + [b - a for _, a, b in rows])[:-1]
+        ctx = SimpleNamespace(q_start=_i32(starts), q_len=_i32(b - a for _, a, b in rows), pos0=_i32(a for _, a, _ in rows),
+                              state_slots=_i32(slots[s] for s, _, _ in rows), num_seqs=len(rows))
+        segments = ops.linear_scan_segments(max(b - a for _, a, b in rows))
+        assert segments == (4, 3, 1)[step]
+        ws = torch.full((len(rows) * segments * H * (dv + 1) * dk,), float("nan"), device=DEV) if segments > 1 else None
+        out = torch.empty(n, H * dv, device=DEV)
+        ops.linear_scan(_dev(cat(0).reshape(n, -1)), _dev(cat(1).reshape(n, -1)), _dev(cat(2).reshape(n, -1)), out, state, ctx, H, dk,
+                        dv, decay=_dev(cat(3).reshape(n, -1)) if gated else None,
+                        head_decay=None if gated else _dev(data[0][3][0, :, 0]), segments=segments, workspace=ws)
+        want = cat(4).reshape(n, H * dv)
+        err = (out.cpu().to(F64) - want).abs().max().item()
+        assert err <= 3e-5 * max(1.0, want.abs().max().item()), (step, err)
+        for s, _, b in rows:
+            done[s] = b
+    assert torch.all(state[2] == -7.0)
+
+
 def test_rotation_of_a_part_of_the_head_and_the_key_scale():
     from glassbox_amd import ops
     torch.manual_seed(3)
@@ -278,6 +320,23 @@ def test_every_way_of_cutting_requests_into_steps(model_dirs, name, dtype):
         assert eng.cache.num_seqs() == 0 and eng.cache.free_state_slots() == 3
         assert all(eng.cache.used_pages(g) == 0 for g in range(len(eng.group_keys)))
         eng.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_whole_and_in_long_portions(model_dirs, dtype):
+    """A prompt of 700 tokens: the recurrent layers cut it into segments, attention crosses its window many times."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, "P")
+    requests = {"long": helpers.random_tokens(211, 700, seed=21), "short": helpers.random_tokens(211, 40, seed=22)}
+    eng = Engine(folder, dtype=dtype, max_tokens=1024, max_seqs=2)
+    _poison(eng)
+    for what, steps in (("whole", helpers.schedule_whole(requests)), ("long portions", helpers.schedule_chunks(requests, (300, 1, 399))),
+                        ("a long portion beside single tokens", [
+                            {"entries": [("short", requests["short"][:39], list(range(39)))], "end": []},
+                            {"entries": [("long", requests["long"], list(range(700))), ("short", requests["short"][39:], [0])],
+                             "end": ["long", "short"]}])):
+        got = helpers.replay(eng, steps)
+        _check(got, folder, requests, dtype, what)
 
 
 def test_the_pool_of_a_windowed_model_holds_windows_not_requests(model_dirs):
