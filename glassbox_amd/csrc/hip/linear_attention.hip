@@ -38,6 +38,7 @@ constexpr int kColsWave = kWave / kLanesCol;
 constexpr int kWaves = 4;
 constexpr int kColsBlock = kColsWave * kWaves;
 constexpr int kThreads = kWaves * kWave;
+constexpr int kPiece = 1024;   // elements of a row a workgroup of the preparing kernels takes
 
 // Sum over the eight lanes of a column (lanes 8c .. 8c+7), by data-parallel moves inside the wave's rows of 16 lanes:
 // neighbours, pairs of neighbours, then the other half of the eight.  Every lane of the eight gets the sum.
@@ -223,13 +224,26 @@ __global__ __launch_bounds__(kThreads) void scan_join_kernel(
   float S0[R];
 #pragma unroll
   for (int m = 0; m < R; ++m) S0[m] = (live && rg * R + m < dk) ? e_row(0)[m] : 0.f;
-  for (int sgm = 1; sgm < sg.seg; ++sgm) {
-    const float* e = e_row(sgm);
-    const float* d = seg_decay + ((cell0 + sgm) * nh + h) * dk + rg * R;
+  constexpr int F = R <= 8 ? 4 : 1;   // segments whose end states are asked for together
+  for (int s0 = 1; s0 < sg.seg; s0 += F) {
+    float e[F][R], d[F][GATED ? R : 1];
 #pragma unroll
-    for (int m = 0; m < R; ++m) {
-      const bool ok = live && rg * R + m < dk;
-      S0[m] = fmaf(GATED ? (ok ? d[m] : 0.f) : whole, S0[m], ok ? e[m] : 0.f);
+    for (int f = 0; f < F; ++f) {
+      const int sgm = min(s0 + f, sg.seg - 1);
+      const float* ep = e_row(sgm);
+      const float* dp = seg_decay + ((cell0 + sgm) * nh + h) * dk + rg * R;
+#pragma unroll
+      for (int m = 0; m < R; ++m) {
+        const bool ok = live && rg * R + m < dk;
+        e[f][m] = ok ? ep[m] : 0.f;
+        if (GATED) d[f][m] = ok ? dp[m] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      if (s0 + f >= sg.seg) break;
+#pragma unroll
+      for (int m = 0; m < R; ++m) S0[m] = fmaf(GATED ? d[f][m] : whole, S0[m], e[f][m]);
     }
   }
 
@@ -259,7 +273,42 @@ __global__ __launch_bounds__(kThreads) void scan_join_kernel(
     if (t0 + kTokens < count) fetch(t0 + kTokens);
     const int here = min(kTokens, count - t0);
     float* orow = out + (size_t)(first + t0) * ((size_t)nh * dv) + (size_t)h * dv + col;
-    for (int j = 0; j < here; ++j) {
+    constexpr int U = R <= 8 ? 4 : R == 16 ? 2 : 1;   // tokens at a time, as in the first kernel
+    // what the first kernel left of these tokens' outputs, asked for before the arithmetic that is added to it
+    float was[kTokens];
+#pragma unroll
+    for (int u = 0; u < kTokens; ++u) was[u] = (rg == 0 && live && u < here) ? orow[(size_t)u * ((size_t)nh * dv)] : 0.f;
+    int j = 0;
+#pragma unroll
+    for (int jj = 0; jj < kTokens; jj += U) {
+      if (jj + U > here) break;
+      j = jj + U;
+      float qq[U][R], aa[GATED ? U : 1][GATED ? R : 1], part[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int m = 0; m < R; ++m) {
+          qq[u][m] = qs[jj + u][rg * R + m];
+          if (GATED) aa[u][m] = ds[jj + u][rg * R + m];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        part[u] = 0.f;
+#pragma unroll
+        for (int m = 0; m < R; ++m) {
+          P[m] *= GATED ? aa[u][m] : decay;
+          part[u] = fmaf(qq[u][m] * P[m], S0[m], part[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) part[u] = sum8(part[u]);
+      if (rg == 0 && live) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) orow[(size_t)(jj + u) * ((size_t)nh * dv)] = was[jj + u] + part[u];
+      }
+    }
+    for (; j < here; ++j) {
       float part = 0.f;
 #pragma unroll
       for (int m = 0; m < R; ++m) {
@@ -287,7 +336,8 @@ __global__ void retention_prep_kernel(const T* __restrict__ proj, int stride, in
                                       float* __restrict__ k32, int nh, int dk, int rot, float k_scale) {
   const int t = blockIdx.x, width = nh * dk, half = rot / 2;
   const T* row = proj + (size_t)t * stride;
-  for (int e = threadIdx.x; e < 2 * width; e += blockDim.x) {
+  // (a workgroup a row and piece of kPiece elements: a step of few rows still spreads over the chip)
+  for (int e = blockIdx.y * kPiece + threadIdx.x; e < min(2 * width, (int)(blockIdx.y + 1) * kPiece); e += blockDim.x) {
     const bool is_k = e >= width;
     const int c = is_k ? e - width : e, d = c % dk;
     const T* src = row + (is_k ? k_off : q_off);
@@ -325,7 +375,7 @@ __global__ void gla_prep_kernel(const T* __restrict__ proj, int stride, int q_of
     for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = to_f(row[low_off + r]);
     __syncthreads();
   }
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  for (int c = blockIdx.y * kPiece + threadIdx.x; c < min(width, (int)(blockIdx.y + 1) * kPiece); c += blockDim.x) {
     q32[(size_t)t * width + c] = to_f(row[q_off + c]) * q_scale;
     k32[(size_t)t * width + c] = to_f(row[k_off + c]);
     float z = 0.f;
@@ -432,13 +482,14 @@ extern "C" int gb_retention_prep(const void* proj, int dtype, int stride, int q_
              n, nh, dk, rot);
   GB_REQUIRE(q_off >= 0 && k_off >= 0 && q_off + nh * dk <= stride && k_off + nh * dk <= stride, "retention_prep: heads beyond the row");
   GB_REQUIRE(rot == 0 || (cosv && sinv), "retention_prep: rotation without tables");
+  GB_REQUIRE(n <= 2147483647 && (2 * nh * dk + kPiece - 1) / kPiece <= 65535, "retention_prep: rows too long for one launch");
   if (n == 0) return 0;
   const int threads = nh * dk >= 512 ? 256 : 128;
   if (dtype == kF32)
-    hipLaunchKernelGGL(retention_prep_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)proj, stride, q_off, k_off,
+    hipLaunchKernelGGL(retention_prep_kernel<float>, dim3(n, (2 * nh * dk + kPiece - 1) / kPiece), dim3(threads), 0, stream, (const float*)proj, stride, q_off, k_off,
                        cosv, sinv, q32, k32, nh, dk, rot, k_scale);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(retention_prep_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)proj, stride, q_off, k_off,
+    hipLaunchKernelGGL(retention_prep_kernel<bf16>, dim3(n, (2 * nh * dk + kPiece - 1) / kPiece), dim3(threads), 0, stream, (const bf16*)proj, stride, q_off, k_off,
                        cosv, sinv, q32, k32, nh, dk, rot, k_scale);
   else
     return fail("retention_prep: unknown dtype %d", dtype);
@@ -456,10 +507,10 @@ extern "C" int gb_gla_prep(const void* proj, int dtype, int stride, int q_off, i
   const int threads = width >= 512 ? 256 : 128;
   const size_t smem = sizeof(float) * rank;
   if (dtype == kF32)
-    hipLaunchKernelGGL(gla_prep_kernel<float>, dim3(n), dim3(threads), smem, stream, (const float*)proj, stride, q_off, k_off,
+    hipLaunchKernelGGL(gla_prep_kernel<float>, dim3(n, (width + kPiece - 1) / kPiece), dim3(threads), smem, stream, (const float*)proj, stride, q_off, k_off,
                        low_off, (const float*)a2, zin, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(gla_prep_kernel<bf16>, dim3(n), dim3(threads), smem, stream, (const bf16*)proj, stride, q_off, k_off,
+    hipLaunchKernelGGL(gla_prep_kernel<bf16>, dim3(n, (width + kPiece - 1) / kPiece), dim3(threads), smem, stream, (const bf16*)proj, stride, q_off, k_off,
                        low_off, (const bf16*)a2, zin, a2_bias, q32, k32, decay, width, rank, q_scale, inv_tau);
   else
     return fail("gla_prep: unknown dtype %d", dtype);

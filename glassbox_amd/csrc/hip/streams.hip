@@ -14,34 +14,89 @@ namespace {
 
 constexpr int kMaxStreams = 8;
 
+// V neighbouring floats as one word where V is 4 (the caller has checked that such words are whole)
+template <int V> __device__ __forceinline__ void load_v(const float* p, float (&v)[V]) {
+  if constexpr (V == 4) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[e] = p[e];
+  }
+}
+template <int V> __device__ __forceinline__ void store_v(float* p, const float (&v)[V]) {
+  if constexpr (V == 4) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) p[e] = v[e];
+  }
+}
+
 // out[r, :] = gamma * u / sqrt(mean(u^2) + eps) with u = sum_s w_in[s] X[s][row] (w_in == nullptr: every weight 1);
-// `rows` (optional) picks the input row of each output row.  One block an output row; `sum` (optional) receives u.
-template <typename G, typename O>
-__global__ void streams_norm_kernel(const float* __restrict__ X, long long stream_stride, int S,
-                                    const float* __restrict__ w_in, const G* __restrict__ gamma,
-                                    const int32_t* __restrict__ rows, O* __restrict__ out, float* __restrict__ sum, int d,
-                                    float eps) {
+// `rows` (optional) picks the input row of each output row.  One block an output row, V columns a thread at a time
+// (V = 4: rows of whole 16-byte words); `sum` (optional) receives u.  With `mix` the streams are first updated by the
+// sublayer before, X'[t] = sum_s mix[s, t] X[s] + w_out[t] y, written back, and u is taken from the new ones: one pass
+// over the streams where the update and the next norm would make two.
+template <typename G, typename O, int V>
+__global__ void streams_norm_kernel(float* __restrict__ X, long long stream_stride, int S, const float* __restrict__ w_in,
+                                    const G* __restrict__ gamma, const int32_t* __restrict__ rows, O* __restrict__ out,
+                                    float* __restrict__ sum, int d, float eps, const float* __restrict__ mix,
+                                    const float* __restrict__ w_out, const float* __restrict__ y) {
   __shared__ float scratch[17];
   extern __shared__ float u[];   // [d]
   const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
-  const float* x0 = X + (size_t)(rows ? rows[r] : r) * d;
+  const size_t row = (size_t)(rows ? rows[r] : r) * d;
   float w[kMaxStreams];
 #pragma unroll
   for (int s = 0; s < kMaxStreams; ++s) w[s] = s < S ? (w_in ? w_in[s] : 1.f) : 0.f;
   float ss = 0.f;
-  for (int c = tid; c < d; c += nt) {
-    float v = 0.f;
+  for (int c = tid * V; c < d; c += nt * V) {
+    float x[kMaxStreams][V], acc[V];
 #pragma unroll
     for (int s = 0; s < kMaxStreams; ++s)
-      if (s < S) v = w_in ? fmaf(w[s], x0[(size_t)s * stream_stride + c], v) : v + x0[(size_t)s * stream_stride + c];
-    u[c] = v;
-    ss = fmaf(v, v, ss);
+      if (s < S) load_v<V>(X + (size_t)s * stream_stride + row + c, x[s]);
+    if (mix) {
+      float yv[V], xn[kMaxStreams][V];
+      load_v<V>(y + row + c, yv);
+#pragma unroll
+      for (int t = 0; t < kMaxStreams; ++t)
+        if (t < S) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < kMaxStreams; ++s)
+              if (s < S) v = fmaf(mix[s * S + t], x[s][e], v);
+            xn[t][e] = fmaf(w_out[t], yv[e], v);
+          }
+          store_v<V>(X + (size_t)t * stream_stride + row + c, xn[t]);
+        }
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s)
+        if (s < S) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) x[s][e] = xn[s][e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      acc[e] = 0.f;
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s)
+        if (s < S) acc[e] = w_in ? fmaf(w[s], x[s][e], acc[e]) : acc[e] + x[s][e];
+      u[c + e] = acc[e];
+      ss = fmaf(acc[e], acc[e], ss);
+    }
   }
   const float total = block_sum(ss, scratch);
   const float scale = 1.0f / sqrtf(total / (float)d + eps);
-  for (int c = tid; c < d; c += nt) {
-    out[(size_t)r * d + c] = from_f<O>(to_f(gamma[c]) * (u[c] * scale));
-    if (sum) sum[(size_t)r * d + c] = u[c];
+  for (int c = tid * V; c < d; c += nt * V) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      out[(size_t)r * d + c + e] = from_f<O>(to_f(gamma[c + e]) * (u[c + e] * scale));
+      if (sum) sum[(size_t)r * d + c + e] = u[c + e];
+    }
   }
 }
 
@@ -73,22 +128,30 @@ __global__ void streams_mix_kernel(float* __restrict__ X, long long stream_strid
 
 extern "C" int gb_streams_max() { return kMaxStreams; }
 
-extern "C" int gb_streams_norm(const float* X, long long stream_stride, int S, const float* w_in, const void* gamma,
+// mix, w_out, y (all or none; not with `rows`): the update of the streams by the sublayer before, done on the way.
+extern "C" int gb_streams_norm(float* X, long long stream_stride, int S, const float* w_in, const void* gamma,
                                int gamma_dtype, const int32_t* rows, void* out, int out_dtype, float* sum, int m, int d,
-                               float eps, hipStream_t stream) {
+                               float eps, const float* mix, const float* w_out, const float* y, hipStream_t stream) {
   GB_REQUIRE(m >= 0 && d > 0 && S >= 1 && S <= kMaxStreams, "streams_norm: bad sizes m=%d d=%d streams=%d (at most %d)", m, d, S,
              kMaxStreams);
   GB_REQUIRE(d <= 16384, "streams_norm: rows of %d columns do not fit a workgroup's memory", d);
+  GB_REQUIRE((mix == nullptr) == (w_out == nullptr) && (mix == nullptr) == (y == nullptr) && (mix == nullptr || rows == nullptr),
+             "streams_norm: the update of the streams takes mix, w_out and y together, and every row in its place");
   if (m == 0) return 0;
-  const int threads = d >= 1024 ? 256 : d >= 256 ? 128 : 64;
+  const int threads = d >= 1024 ? 256 : d >= 256 ? 128 : 64;   // with words of four columns: a pass or two over a row
   const size_t smem = sizeof(float) * d;
+  const bool words = d % 4 == 0 && stream_stride % 4 == 0 && (uintptr_t)X % 16 == 0 && (y == nullptr || (uintptr_t)y % 16 == 0);
 #define GB_SN(G, O)                                                                                                     \
-  hipLaunchKernelGGL((streams_norm_kernel<G, O>), dim3(m), dim3(threads), smem, stream, X, stream_stride, S, w_in,      \
-                     (const G*)gamma, rows, (O*)out, sum, d, eps)
-  if (gamma_dtype == kF32 && out_dtype == kF32) GB_SN(float, float);
-  else if (gamma_dtype == kF32 && out_dtype == kBF16) GB_SN(float, bf16);
-  else if (gamma_dtype == kBF16 && out_dtype == kBF16) GB_SN(bf16, bf16);
-  else if (gamma_dtype == kBF16 && out_dtype == kF32) GB_SN(bf16, float);
+  if (words)                                                                                                            \
+    hipLaunchKernelGGL((streams_norm_kernel<G, O, 4>), dim3(m), dim3(threads), smem, stream, X, stream_stride, S, w_in, \
+                       (const G*)gamma, rows, (O*)out, sum, d, eps, mix, w_out, y);                                     \
+  else                                                                                                                  \
+    hipLaunchKernelGGL((streams_norm_kernel<G, O, 1>), dim3(m), dim3(threads), smem, stream, X, stream_stride, S, w_in, \
+                       (const G*)gamma, rows, (O*)out, sum, d, eps, mix, w_out, y)
+  if (gamma_dtype == kF32 && out_dtype == kF32) { GB_SN(float, float); }
+  else if (gamma_dtype == kF32 && out_dtype == kBF16) { GB_SN(float, bf16); }
+  else if (gamma_dtype == kBF16 && out_dtype == kBF16) { GB_SN(bf16, bf16); }
+  else if (gamma_dtype == kBF16 && out_dtype == kF32) { GB_SN(bf16, float); }
   else return fail("streams_norm: unknown dtypes %d, %d", gamma_dtype, out_dtype);
 #undef GB_SN
   return launched("streams_norm");

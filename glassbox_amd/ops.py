@@ -54,8 +54,8 @@ _SIGS = {
         "gb_scale_rows": [_vp, _f, C.c_longlong, _vp],
     },
     "streams": {
-        # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, stream
-        "gb_streams_norm": [_vp, C.c_longlong, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _f, _vp],
+        # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, mix, w_out, y, stream
+        "gb_streams_norm": [_vp, C.c_longlong, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _f, _vp, _vp, _vp, _vp],
         "gb_streams_mix": [_vp, C.c_longlong, _i, _vp, _vp, _vp, C.c_longlong, _vp],
     },
     "linear_attention": {
@@ -530,10 +530,20 @@ def _streams(X: torch.Tensor, what: str):
 
 
 def streams_norm(X: torch.Tensor, w_in: Optional[torch.Tensor], gamma: torch.Tensor, eps: float, out: torch.Tensor,
-                 rows: Optional[torch.Tensor] = None, total: Optional[torch.Tensor] = None) -> None:
+                 rows: Optional[torch.Tensor] = None, total: Optional[torch.Tensor] = None, update: Optional[tuple] = None) -> None:
     """out[r] = gamma * u / sqrt(mean(u^2) + eps), u = sum_s w_in[s] X[s][rows[r] or r] (``w_in`` None: the plain sum of
-    the streams); ``total`` (float32 [m, d]) receives u as well."""
+    the streams); ``total`` (float32 [m, d]) receives u as well.  ``update=(mix, w_out, y)``: the streams are first
+    updated as ``streams_mix`` does, in the same pass, and u is taken from the new ones (every row, no ``rows``)."""
     _dev(X, w_in, gamma, out, rows, total)
+    mix = w_out = y = None
+    if update is not None:
+        mix, w_out, y = update
+        _dev(mix, w_out, y)
+        S0, n0, d0 = X.shape
+        if rows is not None or out.shape[0] != n0 or y.dtype != torch.float32 or y.shape != (n0, d0) or not y.is_contiguous() \
+                or mix.dtype != torch.float32 or mix.shape != (S0, S0) or not mix.is_contiguous() \
+                or w_out.dtype != torch.float32 or w_out.numel() != S0 or not w_out.is_contiguous():
+            raise KernelError("streams_norm: update=(mix [S, S], w_out [S], y [n, d]) in float32, on every row")
     S, n, d = _streams(X, "streams_norm")
     m = out.shape[0]
     if out.shape != (m, d) or not out.is_contiguous() or gamma.numel() != d or not gamma.is_contiguous():
@@ -547,7 +557,7 @@ def streams_norm(X: torch.Tensor, w_in: Optional[torch.Tensor], gamma: torch.Ten
     _i32(rows, "rows", m)
     lib = _lib("streams")
     _launch(lib, lib.gb_streams_norm, _p(X), X.stride(0), S, _p(w_in), _p(gamma), dtype_code(gamma), _p(rows), _p(out),
-            dtype_code(out), _p(total), m, d, float(eps), _stream())
+            dtype_code(out), _p(total), m, d, float(eps), _p(mix), _p(w_out), _p(y), _stream())
 
 
 def streams_mix(X: torch.Tensor, mix: torch.Tensor, w_out: torch.Tensor, y: torch.Tensor) -> None:

@@ -169,8 +169,9 @@ class GatedLinearAttention(_LinearMixer):
         decay = ctx.buffer("lin_decay", (n, self.qk_dim), torch.float32)
         low_off, rank = 2 * self.qk_dim + 2 * self.v_dim, self.w_a2.shape[1]
         z = None
-        if n > ops.FUSED_NORM_MAX_ROWS and (ctx.dtype == torch.float32 or (rank % 8 == 0 and low_off % 8 == 0)):
-            # many rows: the second matrix of the decay's projection as a product of its own (few rows: inside the kernel)
+        if ctx.dtype == torch.float32 or (rank % 8 == 0 and low_off % 8 == 0):
+            # the second matrix of the decay's projection as a product of its own (sizes that a bfloat16 product does not
+            # take: inside the kernel)
             z = ctx.buffer("lin_z", (n, self.qk_dim), torch.float32)
             ops.gemm(proj[:, low_off:low_off + rank], self.w_a2, z)
         ops.gla_prep(proj, 0, self.qk_dim, low_off, self.w_a2, self.a2_bias, q32, k32, decay,

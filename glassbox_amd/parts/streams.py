@@ -15,7 +15,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import Block, CacheSpec, FeedForward, LayerCache, Mixer, Part, StateSpec, TensorSpec
+from .base import Block, CacheSpec, FeedForward, LayerCache, Mixer, Normed, Part, StateSpec, TensorSpec
 from .norm import RMSNorm
 
 
@@ -82,16 +82,36 @@ class StreamsBlock(Block):
     def state_spec(self) -> Optional[StateSpec]:
         return self.mixer.state_spec
 
-    def forward(self, ctx, x, cache: Optional[LayerCache]):
-        """``x``: the streams, float32 [streams, n, width], updated in place."""
+    def entry_norm(self, ctx, n: int):
+        """What the block before needs to do this block's first norm in the pass that updates the streams with its
+        last sublayer: ``(in weights, gamma, eps)`` (``forward(..., pre=)`` then takes the rows it made)."""
+        return (self.hc1_in, self.mixer_norm.weight, self.mixer_norm.eps) if ctx.tuned else None
+
+    def forward(self, ctx, x, cache: Optional[LayerCache], pre=None, emit=None):
+        """``x``: the streams, float32 [streams, n, width], updated in place.  ``pre``: a ``Normed`` with the rows of this
+        block's first norm, from the block before; ``emit``: the ``entry_norm`` of the block after, whose rows this
+        block then returns as a ``Normed``.  An update of the streams and the norm that reads them next are one kernel."""
         n, width = x.shape[1], x.shape[2]
         y = ctx.buffer("streams_y", (n, width), torch.float32)
         h = ctx.buffer("h", (n, width), ctx.dtype)
-        ops.streams_norm(x, self.hc1_in, self.mixer_norm.weight, self.mixer_norm.eps, h)
+        if isinstance(pre, Normed):
+            h = pre.rows
+        else:
+            ops.streams_norm(x, self.hc1_in, self.mixer_norm.weight, self.mixer_norm.eps, h)
         self.mixer.forward(ctx, h, y, cache, store=True)
-        ops.streams_mix(x, self.hc1_mix, self.hc1_out, y)
+        last = (self.hc1_mix, self.hc1_out, y)
         if self.ffn is not None:
-            ops.streams_norm(x, self.hc2_in, self.ffn_norm.weight, self.ffn_norm.eps, h)
+            if ctx.tuned:
+                ops.streams_norm(x, self.hc2_in, self.ffn_norm.weight, self.ffn_norm.eps, h, update=last)
+            else:
+                ops.streams_mix(x, *last)
+                ops.streams_norm(x, self.hc2_in, self.ffn_norm.weight, self.ffn_norm.eps, h)
             self.ffn.forward(ctx, h, y, store=True)
-            ops.streams_mix(x, self.hc2_mix, self.hc2_out, y)
+            last = (self.hc2_mix, self.hc2_out, y)
+        if emit is not None:
+            w_in, gamma, eps = emit
+            handed = ctx.buffer("h_next", (n, width), ctx.dtype)
+            ops.streams_norm(x, w_in, gamma, eps, handed, update=last)
+            return Normed(handed)
+        ops.streams_mix(x, *last)
         return None

@@ -174,9 +174,16 @@ def test_streams_kernels():
         picked = torch.empty(2, d, device=DEV)
         ops.streams_norm(Xd, None, _dev(gamma), 1e-5, picked, rows=rows)
         assert (picked.cpu().to(F64) - ps.rms(f(X).sum(0)[[n - 1, 0]], 1e-5, f(gamma))).abs().max() < 1e-5
+        again = Xd.clone()
         ops.streams_mix(Xd, _dev(mix), _dev(w_out), _dev(y))
         want = torch.stack([sum(f(mix)[s, t] * f(X)[s] for s in range(S)) + f(w_out)[t] * f(y) for t in range(S)])
         assert (Xd.cpu().to(F64) - want).abs().max() < 1e-5
+        # the update and the norm that reads the streams next, in one pass
+        h2 = torch.empty(n, d, device=DEV)
+        ops.streams_norm(again, _dev(w_in), _dev(gamma), 1e-5, h2, update=(_dev(mix), _dev(w_out), _dev(y)))
+        assert (again.cpu().to(F64) - want).abs().max() < 1e-5
+        u2 = sum(f(w_in)[s] * want[s] for s in range(S))
+        assert (h2.cpu().to(F64) - ps.rms(u2, 1e-5, f(gamma))).abs().max() < 2e-5
 
 
 # ------------------------------------------------------------------------------------------ attention
