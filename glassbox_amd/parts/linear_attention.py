@@ -64,10 +64,18 @@ class _LinearMixer(Mixer):
             parts = list(parts) + [torch.zeros((8 - rows % 8, parts[0].shape[1]), dtype=parts[0].dtype, device=parts[0].device)]
         return torch.cat(parts, 0)
 
-    def _project(self, ctx, h):
+    def _project(self, ctx, h, tail: int = 0):
+        """The stacked input product.  ``tail``: the last so many rows of the stacked matrix (beyond a multiple of the
+        product's tiles they would cost a step of many rows a second round of tiles) go through a product of their own."""
         n = h.shape[0]
-        proj = ctx.buffer("lin_proj", (n, self.w_in.shape[0]), ctx.dtype)
-        ops.gemm(h, self.w_in, proj, workspace=split_workspace(ctx, n, self.w_in.shape[0], self.width))
+        rows = self.w_in.shape[0]
+        proj = ctx.buffer("lin_proj", (n, rows), ctx.dtype)
+        if tail and n > ops.ROPE_PRODUCT_MAX_ROWS:
+            main = rows - tail
+            ops.gemm(h, self.w_in[:main], proj[:, :main], workspace=split_workspace(ctx, n, main, self.width))
+            ops.gemm(h, self.w_in[main:], proj[:, main:], workspace=split_workspace(ctx, n, tail, self.width))
+        else:
+            ops.gemm(h, self.w_in, proj, workspace=split_workspace(ctx, n, rows, self.width))
         return proj
 
     def _finish(self, ctx, proj, q32, k32, residual, cache, store, norm_weight, decay=None, head_decay=None):
@@ -163,7 +171,9 @@ class GatedLinearAttention(_LinearMixer):
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
         """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
         n = h.shape[0]
-        proj = self._project(ctx, h)
+        main = 2 * self.qk_dim + 2 * self.v_dim
+        # (the narrow rows of the decay and the filling rows behind them, where the rest is whole words)
+        proj = self._project(ctx, h, tail=self.w_in.shape[0] - main if main % 8 == 0 else 0)
         q32 = ctx.buffer("lin_q", (n, self.qk_dim), torch.float32)
         k32 = ctx.buffer("lin_k", (n, self.qk_dim), torch.float32)
         decay = ctx.buffer("lin_decay", (n, self.qk_dim), torch.float32)
