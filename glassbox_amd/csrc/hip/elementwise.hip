@@ -658,6 +658,57 @@ __global__ __launch_bounds__(4 * kWave) void qk_norm_store_kernel(T* __restrict_
   }
 }
 
+// The same for a step of many rows whose values stay in the rows (v_off >= 0): sixteen lanes a (token, head), a lane
+// 16-byte words of the head (heads of whole words, up to 256 dimensions), sixteen heads a workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rows_kernel(T* __restrict__ qk, int stride, const float* __restrict__ bias_q,
+                                                         const float* __restrict__ bias_k, const float* __restrict__ w_q,
+                                                         const float* __restrict__ w_k, float eps, int nh, int nkv, int hd,
+                                                         int v_off, int pairs) {
+  constexpr int E = 16 / (int)sizeof(T);        // elements a word
+  constexpr int IT = 256 / (16 * E);            // words a lane at most
+  typedef T word __attribute__((ext_vector_type(E)));
+  const int pair = blockIdx.x * 16 + threadIdx.x / 16, li = threadIdx.x % 16;
+  const bool live = pair < pairs;
+  const int t = live ? pair / (nh + nkv) : 0, h = live ? pair % (nh + nkv) : 0;
+  const bool is_key = h >= nh;
+  T* row = qk + (size_t)t * stride + (size_t)h * hd;
+  const float* bias = is_key ? (bias_k ? bias_k + (size_t)(h - nh) * hd : nullptr) : (bias_q ? bias_q + (size_t)h * hd : nullptr);
+  const float* w = is_key ? w_k : w_q;
+  float x[IT][E];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int d0 = (it * 16 + li) * E;
+    if (live && d0 < hd) {
+      const word v = *reinterpret_cast<const word*>(row + d0);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        // what the projection gives in this type, bias included, is the value and the norm's operand alike
+        x[it][e] = to_f(from_f<T>(to_f(v[e]) + (bias ? bias[d0 + e] : 0.f)));
+        ss = fmaf(x[it][e], x[it][e], ss);
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) ss += __shfl_xor(ss, o, kWave);
+  const float s = w ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.0f;
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int d0 = (it * 16 + li) * E;
+    if (live && d0 < hd) {
+      word y, raw;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        y[e] = from_f<T>(w ? w[d0 + e] * (x[it][e] * s) : x[it][e]);
+        raw[e] = from_f<T>(x[it][e]);
+      }
+      *reinterpret_cast<word*>(row + d0) = y;
+      if (is_key) *reinterpret_cast<word*>(qk + (size_t)t * stride + v_off + (size_t)(h - nh) * hd + d0) = raw;
+    }
+  }
+}
+
 extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bias_q, const float* bias_k, const float* w_q,
                                 const float* w_k, float eps, const int32_t* slots, void* k_pages, void* v_pages, int n,
                                 int nh, int nkv, int hd, int page_size, int v_off, hipStream_t stream) {
@@ -670,6 +721,18 @@ extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bi
   GB_REQUIRE((long long)n * (nh + nkv) < (1ll << 31), "qk_norm_store: too many (token, head) pairs");
   if (n == 0) return 0;
   const int pairs = n * (nh + nkv);
+  const int word = dtype == kF32 ? 4 : 8;
+  if (v_off >= 0 && hd % word == 0 && stride % word == 0 && v_off % word == 0 && (uintptr_t)qk % 16 == 0 &&
+      (dtype == kF32 || dtype == kBF16)) {
+    const dim3 rows_grid((unsigned)((pairs + 15) / 16));
+    if (dtype == kF32)
+      hipLaunchKernelGGL(qk_norm_rows_kernel<float>, rows_grid, dim3(256), 0, stream, (float*)qk, stride, bias_q, bias_k, w_q, w_k,
+                         eps, nh, nkv, hd, v_off, pairs);
+    else
+      hipLaunchKernelGGL(qk_norm_rows_kernel<bf16>, rows_grid, dim3(256), 0, stream, (bf16*)qk, stride, bias_q, bias_k, w_q, w_k,
+                         eps, nh, nkv, hd, v_off, pairs);
+    return launched("qk_norm_store");
+  }
   const dim3 grid((unsigned)((pairs + 3) / 4));
   if (dtype == kF32)
     hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, dim3(4 * kWave), 0, stream, (float*)qk, stride, bias_q, bias_k, w_q, w_k,

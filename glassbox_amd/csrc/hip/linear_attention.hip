@@ -412,6 +412,48 @@ __global__ __launch_bounds__(4 * kWave) void head_norm_gate_kernel(const float* 
   }
 }
 
+// The same with sixteen lanes a (token, head), a lane words of four values, sixteen heads a workgroup: for every dv that
+// is a multiple of 4 up to 256, whatever the number of rows (a head's sum is then added up in one order always).
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_words_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                                 int gate_stride, const float* __restrict__ w,
+                                                                 T* __restrict__ out, int nh, int dv, float eps, int pairs) {
+  constexpr int IT = 4;
+  typedef T quad __attribute__((ext_vector_type(4)));
+  const int pair = blockIdx.x * 16 + threadIdx.x / 16, li = threadIdx.x % 16;
+  const bool live = pair < pairs;
+  const int t = live ? pair / nh : 0, h = live ? pair % nh : 0;
+  const float* orow = o + ((size_t)t * nh + h) * dv;
+  f32x4 x[IT];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int d0 = (it * 16 + li) * 4;
+    if (live && d0 < dv) {
+      x[it] = *reinterpret_cast<const f32x4*>(orow + d0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss = fmaf(x[it][e], x[it][e], ss);
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) ss += __shfl_xor(ss, off, kWave);
+  const float s = 1.0f / sqrtf(ss / (float)dv + eps);
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int d0 = (it * 16 + li) * 4;
+    if (live && d0 < dv) {
+      const quad g4 = *reinterpret_cast<const quad*>(gate + (size_t)t * gate_stride + (size_t)h * dv + d0);
+      quad y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float g = to_f(g4[e]);
+        y[e] = from_f<T>(((w ? w[d0 + e] : 1.0f) * (x[it][e] * s)) * (g / (1.0f + expf(-g))));
+      }
+      *reinterpret_cast<quad*>(out + ((size_t)t * nh + h) * dv + d0) = y;
+    }
+  }
+}
+
 template <typename T, bool GATED>
 int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const float* k, const float* a, const float* head_decay,
                 const void* v, int v_stride, float* out, float* state, const int32_t* q_start, const int32_t* q_len,
@@ -522,6 +564,18 @@ extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, in
   GB_REQUIRE(n >= 0 && nh > 0 && dv > 0 && gate_stride >= nh * dv, "head_norm_gate: bad sizes n=%d heads=%d dv=%d", n, nh, dv);
   GB_REQUIRE((long long)n * nh < (1ll << 31), "head_norm_gate: too many (token, head) pairs");
   if (n == 0) return 0;
+  const int pairs = n * nh, gw = dtype == kF32 ? 16 : 8;   // (a gate word of four values: 16 or 8 bytes)
+  if (dv % 4 == 0 && dv <= 256 && gate_stride % 4 == 0 && (uintptr_t)gate % gw == 0 && (uintptr_t)o % 16 == 0 &&
+      (uintptr_t)out % gw == 0 && (dtype == kF32 || dtype == kBF16)) {
+    const dim3 grid((unsigned)((pairs + 15) / 16));
+    if (dtype == kF32)
+      hipLaunchKernelGGL(head_norm_gate_words_kernel<float>, grid, dim3(256), 0, stream, o, (const float*)gate, gate_stride, w,
+                         (float*)out, nh, dv, eps, pairs);
+    else
+      hipLaunchKernelGGL(head_norm_gate_words_kernel<bf16>, grid, dim3(256), 0, stream, o, (const bf16*)gate, gate_stride, w,
+                         (bf16*)out, nh, dv, eps, pairs);
+    return launched("head_norm_gate");
+  }
   if (dtype == kF32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3((unsigned)((n * nh + 3) / 4)), dim3(4 * kWave), 0, stream, o,
                        (const float*)gate, gate_stride, w, (float*)out, nh, dv, eps, n * nh);

@@ -147,13 +147,14 @@ def test_decays_of_key_channels_and_the_gated_head_norm():
     assert (decay.cpu().to(F64) - want).abs().max() < 2e-6 and 0.0 < float(decay.min()) and float(decay.max()) <= 1.0
     assert (q32.cpu().to(F64) - 0.5 * qk[:, :width].float().to(F64)).abs().max() < 1e-6
     assert torch.equal(k32.cpu(), qk[:, width:].float())
-    H, dv, eps = 3, 20, 1e-3
-    o, gate, wn = torch.randn(T, H, dv, dtype=F64) * 5, torch.randn(T, H * dv, dtype=F64), torch.rand(dv, dtype=F64) + 0.5
-    for w in (None, wn):
-        out = torch.empty(T, H * dv, device=DEV)
-        ops.head_norm_gate(_dev(o.reshape(T, -1)), _dev(gate), None if w is None else _dev(w), out, H, dv, eps)
-        want = ps.rms(o.float().to(F64), eps, None if w is None else w.float().to(F64)).reshape(T, -1) * ps.silu(gate.float().to(F64))
-        assert (out.cpu().to(F64) - want).abs().max() < 1e-5
+    eps = 1e-3
+    for T, H, dv in ((9, 3, 20), (70, 3, 20), (70, 2, 72), (65, 1, 7)):   # (few rows and many take different kernels)
+        o, gate, wn = torch.randn(T, H, dv, dtype=F64) * 5, torch.randn(T, H * dv, dtype=F64), torch.rand(dv, dtype=F64) + 0.5
+        for w in (None, wn):
+            out = torch.empty(T, H * dv, device=DEV)
+            ops.head_norm_gate(_dev(o.reshape(T, -1)), _dev(gate), None if w is None else _dev(w), out, H, dv, eps)
+            want = ps.rms(o.float().to(F64), eps, None if w is None else w.float().to(F64)).reshape(T, -1) * ps.silu(gate.float().to(F64))
+            assert (out.cpu().to(F64) - want).abs().max() < 1e-5, (T, H, dv)
 
 
 # ------------------------------------------------------------------------------------------ streams
