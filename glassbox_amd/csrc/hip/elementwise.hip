@@ -682,10 +682,16 @@ __global__ __launch_bounds__(256) void qk_norm_rows_kernel(T* __restrict__ qk, i
     const int d0 = (it * 16 + li) * E;
     if (live && d0 < hd) {
       const word v = *reinterpret_cast<const word*>(row + d0);
+      float b[E];
+#pragma unroll
+      for (int e4 = 0; e4 < E; e4 += 4) {   // (bias and weight as words of four floats: hd is a multiple of E)
+        const f32x4 b4 = bias ? *reinterpret_cast<const f32x4*>(bias + d0 + e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        b[e4] = b4[0]; b[e4 + 1] = b4[1]; b[e4 + 2] = b4[2]; b[e4 + 3] = b4[3];
+      }
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // what the projection gives in this type, bias included, is the value and the norm's operand alike
-        x[it][e] = to_f(from_f<T>(to_f(v[e]) + (bias ? bias[d0 + e] : 0.f)));
+        x[it][e] = to_f(from_f<T>(to_f(v[e]) + b[e]));
         ss = fmaf(x[it][e], x[it][e], ss);
       }
     }
@@ -698,9 +704,15 @@ __global__ __launch_bounds__(256) void qk_norm_rows_kernel(T* __restrict__ qk, i
     const int d0 = (it * 16 + li) * E;
     if (live && d0 < hd) {
       word y, raw;
+      float g[E];
+#pragma unroll
+      for (int e4 = 0; e4 < E; e4 += 4) {
+        const f32x4 g4 = w ? *reinterpret_cast<const f32x4*>(w + d0 + e4) : f32x4{1.f, 1.f, 1.f, 1.f};
+        g[e4] = g4[0]; g[e4 + 1] = g4[1]; g[e4 + 2] = g4[2]; g[e4 + 3] = g4[3];
+      }
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        y[e] = from_f<T>(w ? w[d0 + e] * (x[it][e] * s) : x[it][e]);
+        y[e] = from_f<T>(w ? g[e] * (x[it][e] * s) : x[it][e]);
         raw[e] = from_f<T>(x[it][e]);
       }
       *reinterpret_cast<word*>(row + d0) = y;
@@ -722,7 +734,9 @@ extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bi
   if (n == 0) return 0;
   const int pairs = n * (nh + nkv);
   const int word = dtype == kF32 ? 4 : 8;
-  if (v_off >= 0 && hd % word == 0 && stride % word == 0 && v_off % word == 0 && (uintptr_t)qk % 16 == 0 &&
+  const bool vectors = (!bias_q || (uintptr_t)bias_q % 16 == 0) && (!bias_k || (uintptr_t)bias_k % 16 == 0) &&
+                       (!w_q || (uintptr_t)w_q % 16 == 0) && (!w_k || (uintptr_t)w_k % 16 == 0);
+  if (v_off >= 0 && vectors && hd % word == 0 && stride % word == 0 && v_off % word == 0 && (uintptr_t)qk % 16 == 0 &&
       (dtype == kF32 || dtype == kBF16)) {
     const dim3 rows_grid((unsigned)((pairs + 15) / 16));
     if (dtype == kF32)
