@@ -4,6 +4,8 @@
 // through its norm, and its output y [tokens, width] (float32) goes back into all of them at once:
 //   X'[t] = sum_s mix[s, t] X[s] + w_out[t] y     (mix is indexed [from, to]) .
 // At the end the model's norm reads sum_s X[s].  All sums are 32-bit, streams added in ascending s.
+#include <algorithm>
+
 #include "common.h"
 
 using namespace gb;
@@ -138,9 +140,11 @@ extern "C" int gb_streams_norm(float* X, long long stream_stride, int S, const f
   GB_REQUIRE((mix == nullptr) == (w_out == nullptr) && (mix == nullptr) == (y == nullptr) && (mix == nullptr || rows == nullptr),
              "streams_norm: the update of the streams takes mix, w_out and y together, and every row in its place");
   if (m == 0) return 0;
-  const int threads = d >= 1024 ? 256 : d >= 256 ? 128 : 64;   // with words of four columns: a pass or two over a row
   const size_t smem = sizeof(float) * d;
   const bool words = d % 4 == 0 && stream_stride % 4 == 0 && (uintptr_t)X % 16 == 0 && (y == nullptr || (uintptr_t)y % 16 == 0);
+  // a thread for every word of the row, up to 1,024: all of a row's loads are asked for at once
+  const int per = words ? 4 : 1;
+  const int threads = std::min(1024, std::max(64, ((d + per - 1) / per + 63) / 64 * 64));
 #define GB_SN(G, O)                                                                                                     \
   if (words)                                                                                                            \
     hipLaunchKernelGGL((streams_norm_kernel<G, O, 4>), dim3(m), dim3(threads), smem, stream, X, stream_stride, S, w_in, \
