@@ -48,8 +48,20 @@ CASES: Dict[str, dict] = {
                                         "mask": {"size": 9, "keep_first": 3}}, "mlp": {"kind": "dense", "ff": 30}},
         {"type": "gla", "mixer": {"heads": 2, "dim": 12, "vdim": 5, "tau": 2.5, "rank": 3}, "mlp": None},
     ]),
+    # heads that the matrix-core attention kernels do not take (40 and 24 dimensions: the plain kernel in bfloat16 too),
+    # four streams, a decay's middle that is no multiple of 8, a window shorter than a page
+    "S": dict(architecture="Sagalorn", vocab=160, width=80, streams=4, logit_scale=1.5, embedding={"scale": 2.0},
+              norm={"eps": 2e-5}, loop={"start": 0, "stop": 3, "times": 2}, layers=[
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 40, "vdim": 40, "scale": 0.5,
+                                        "mask": {"size": 11, "keep_first": 2}}, "mlp": None},
+        {"type": "gla", "mixer": {"heads": 2, "dim": 40, "vdim": 24, "tau": 8.0, "rank": 12}, "mlp": {"kind": "dense", "ff": 56}},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 4, "dim": 24, "vdim": 24, "scale": 0.7,
+                                        "mask": {"size": 50, "keep_first": 17}}, "mlp": None},
+        {"type": "retention", "mixer": {"heads": 5, "dim": 16, "vdim": 16, "decay": [0.7, 0.9, 0.95, 0.99, 0.999],
+                                        "rot": {"dims": 16, "base": 1000.0}}, "mlp": None},
+    ]),
 }
-BF16_CASES = ("P", "Q", "R")
+BF16_CASES = ("P", "Q", "R", "S")
 
 
 def folder_of(base: str, name: str, seed: int = 0, std: float = 0.05) -> str:
