@@ -759,6 +759,51 @@ extern "C" int gb_qk_norm_store(void* qk, int dtype, int stride, const float* bi
   return launched("qk_norm_store");
 }
 
+// ------------------------------------------------------------------------ plain product
+// c (+)= a . w^T for operands of any size and alignment, one thread a cell, tiles of 16 x 16 through LDS, 32-bit sums in
+// ascending k.  For the products of a model whose sizes the matrix-core kernels do not take (inner sizes that are no
+// multiple of 8 in bfloat16); nothing here is tuned.
+template <typename T, typename O>
+__global__ __launch_bounds__(256) void gemm_plain_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, int ldw,
+                                                       O* __restrict__ c, int ldc, int M, int N, int K, int accumulate) {
+  __shared__ float As[16][17], Ws[16][17];
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  const int m = blockIdx.y * 16 + ty, n = blockIdx.x * 16 + tx, wn = blockIdx.x * 16 + ty;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    As[ty][tx] = (m < M && k0 + tx < K) ? to_f(a[(size_t)m * lda + k0 + tx]) : 0.f;
+    Ws[ty][tx] = (wn < N && k0 + tx < K) ? to_f(w[(size_t)wn * ldw + k0 + tx]) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) acc = fmaf(As[ty][kk], Ws[tx][kk], acc);
+    __syncthreads();
+  }
+  if (m < M && n < N) {
+    O* cell = c + (size_t)m * ldc + n;
+    *cell = from_f<O>(accumulate ? to_f(*cell) + acc : acc);
+  }
+}
+
+extern "C" int gb_gemm_plain(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int dtype, int c_dtype, int M,
+                             int N, int K, int accumulate, hipStream_t stream) {
+  GB_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldw >= K && ldc >= N, "gemm_plain: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M == 0) return 0;
+  const dim3 grid((N + 15) / 16, (M + 15) / 16);
+  GB_REQUIRE(grid.y <= 65535, "gemm_plain: M=%d needs more than 65535 row tiles", M);
+  if (dtype == kBF16 && c_dtype == kBF16)
+    hipLaunchKernelGGL((gemm_plain_kernel<bf16, bf16>), grid, dim3(256), 0, stream, (const bf16*)a, lda, (const bf16*)w, ldw,
+                       (bf16*)c, ldc, M, N, K, accumulate);
+  else if (dtype == kBF16 && c_dtype == kF32)
+    hipLaunchKernelGGL((gemm_plain_kernel<bf16, float>), grid, dim3(256), 0, stream, (const bf16*)a, lda, (const bf16*)w, ldw,
+                       (float*)c, ldc, M, N, K, accumulate);
+  else if (dtype == kF32 && c_dtype == kF32)
+    hipLaunchKernelGGL((gemm_plain_kernel<float, float>), grid, dim3(256), 0, stream, (const float*)a, lda, (const float*)w, ldw,
+                       (float*)c, ldc, M, N, K, accumulate);
+  else
+    return fail("gemm_plain: operand and result types %d, %d", dtype, c_dtype);
+  return launched("gemm_plain");
+}
+
 // ------------------------------------------------------------------------ scale
 // x *= s   (float32: logits that a model scales)
 __global__ void scale_rows_kernel(float* __restrict__ x, float s, long long count) {
@@ -797,3 +842,4 @@ GB_TAPED(gb_copy_rows)
 GB_TAPED(gb_qk_norm_store)
 GB_TAPED(gb_add_bias)
 GB_TAPED(gb_scale_rows)
+GB_TAPED(gb_gemm_plain)

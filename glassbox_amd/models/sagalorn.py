@@ -45,7 +45,7 @@ def build_sagalorn(cfg: SagalornConfig) -> DecoderModel:
     blocks = []
     for layer in cfg.layers:
         mixer = _mixer(cfg, layer)
-        ffn = SwiGLU(d, layer["mlp"]["ff"]) if layer["mlp"] is not None else None
+        ffn = SwiGLU(d, layer["mlp"]["ff"], any_size=True) if layer["mlp"] is not None else None
         if cfg.streams is not None:
             blocks.append(StreamsBlock(cfg.streams, RMSNorm(d, eps), mixer, RMSNorm(d, eps) if ffn is not None else None, ffn))
         elif ffn is not None:
@@ -55,7 +55,7 @@ def build_sagalorn(cfg: SagalornConfig) -> DecoderModel:
     schedule = [LayerCall(block=b, cache=c) for c, b in enumerate(cfg.layer_order())]
     final = StreamsSumNorm(d, eps) if cfg.streams is not None else RMSNorm(d, eps)
     return DecoderModel(cfg, Embedding(cfg.vocab, d, cfg.embedding_scale), blocks, schedule, final,
-                        LMHead(cfg.vocab, d, scale=cfg.logit_scale), names=("embed", "l{}", "final.norm", "head"),
+                        LMHead(cfg.vocab, d, scale=cfg.logit_scale, any_size=True), names=("embed", "l{}", "final.norm", "head"),
                         sources=_source, streams=cfg.streams,
                         arg_keys={"width": "width", "intermediate": "layers[].mlp.ff", "dim": "layers[].mixer.dim",
                                   "heads * dim": "layers[].mixer.heads, dim", "heads * vdim": "layers[].mixer.heads, vdim",

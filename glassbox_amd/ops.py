@@ -52,6 +52,8 @@ _SIGS = {
         "gb_qk_norm_store": [_vp, _i, _i, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
         "gb_add_bias": [_vp, _vp, _i, _i, _vp],
         "gb_scale_rows": [_vp, _f, C.c_longlong, _vp],
+        # a, lda, w, ldw, c, ldc, operand dtype, result dtype, M, N, K, accumulate, stream
+        "gb_gemm_plain": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     },
     "streams": {
         # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, mix, w_out, y, stream
@@ -823,6 +825,30 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                      workspace.numel() if workspace is not None else 0, _stream())
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
+
+
+def gemm_takes(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm`` takes these operands: 32-bit ones always; bfloat16 ones whose inner size is a multiple of 8 and
+    whose rows begin at 16-byte words."""
+    if a.dtype != torch.bfloat16:
+        return True
+    return (a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out (+)= a . w^T by the plain kernel (one thread a cell): operands of one type, bfloat16 or float32, of any size and
+    alignment; out in the operands' type or float32.  What a model's odd sizes fall back to; ``gemm`` is the product."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or out.shape != (M, N) or a.dtype != w.dtype:
+        raise KernelError(f"gemm_plain: shapes or types do not match: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if accumulate and out.dtype != torch.float32:
+        raise KernelError("gemm_plain: accumulation is into a 32-bit result")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_gemm_plain, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(out), _rows(out, "out"), dtype_code(a),
+            dtype_code(out), M, N, K, 1 if accumulate else 0, _stream())
 
 
 ROPE_PRODUCT_MAX_ROWS = 64

@@ -16,7 +16,7 @@ import torch
 
 from .. import ops
 from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target,
-                   needs_multiple_of_8, split_workspace)
+                   needs_multiple_of_8, product, split_workspace)
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, n_heads: int, scale: float,
@@ -201,7 +201,7 @@ class TiedValueAttention(Mixer):
         return [self.wqk, self.wo]
 
     def problems(self, dtype, page_size):
-        out = needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "heads * dim", self.q_dim)
+        out = []   # (sizes that the matrix-core products do not take go through the plain product)
         if self.head_dim > ops.MAX_HEAD_DIM:
             out.append(("dim", f"{self.head_dim} is above {ops.MAX_HEAD_DIM}, the largest head the attention kernels take"))
         return out
@@ -217,19 +217,19 @@ class TiedValueAttention(Mixer):
             # values to their pages in whole lines does the cache write (no rotation)
             rows = ctx.buffer("qkv", (n, self.q_dim + 2 * self.kv_dim), ctx.dtype)
             qk = rows[:, :self.q_dim + self.kv_dim]
-            ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
+            product(ctx, h, self.wqk, qk)
             ops.qk_norm_store(rows, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, None, None, None,
                               self.n_heads, self.n_kv_heads, self.head_dim, values_in_rows=True)
             ops.rope_store(rows, None, None, slots, cache.k_pages, cache.v_pages, self.n_heads, self.n_kv_heads,
                            self.head_dim, rotate=False, portions=ctx.portions())
         else:
             qk = ctx.buffer("qk", (n, self.q_dim + self.kv_dim), ctx.dtype)
-            ops.gemm(h, self.wqk, qk, workspace=split_workspace(ctx, n, self.q_dim + self.kv_dim, self.width))
+            product(ctx, h, self.wqk, qk)
             ops.qk_norm_store(qk, self.bias_q, self.bias_k, self.norm_q, self.norm_k, self.eps, slots,
                               cache.k_pages if slots is not None else None, cache.v_pages if slots is not None else None,
                               self.n_heads, self.n_kv_heads, self.head_dim)
         att = ctx.buffer("att", (n, self.q_dim), ctx.dtype)
         paged_attention(ctx, qk[:, :self.q_dim], att, cache, self.n_heads, self.scale, self.window, self.keep_first)
-        ops.gemm(att, self.wo, residual, accumulate=not store, workspace=split_workspace(ctx, n, self.width, self.q_dim))
+        product(ctx, att, self.wo, residual, accumulate=not store)
         if self.bias_o is not None:
             ops.add_bias(residual, self.bias_o)

@@ -242,6 +242,17 @@ def split_workspace(ctx, n: int, out_features: int, in_features: int):
     return ctx.buffer("gemm_split", (floats,), torch.float32) if floats else None
 
 
+def product(ctx, a, w, out, accumulate: bool = False) -> None:
+    """``out (+)= a . w^T`` for parts that take models of any sizes: ``ops.gemm`` (with a workspace where it would divide
+    k), or, for bfloat16 operands that it does not take (an inner size that is no multiple of 8, rows that do not begin
+    at 16-byte words), the plain product."""
+    from .. import ops
+    if ops.gemm_takes(a, w):
+        ops.gemm(a, w, out, accumulate=accumulate, workspace=split_workspace(ctx, a.shape[0], w.shape[0], a.shape[1]))
+    else:
+        ops.gemm_plain(a, w, out, accumulate=accumulate)
+
+
 class Mixer(Part):
     cache_spec: Optional[CacheSpec] = None
     state_spec: Optional[StateSpec] = None

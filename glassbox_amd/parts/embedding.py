@@ -8,7 +8,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import Part, TensorSpec, needs_multiple_of_8
+from .base import Part, TensorSpec, needs_multiple_of_8, product
 
 
 class Embedding(Part):
@@ -33,8 +33,9 @@ class LMHead(Part):
     """logits = rows . W^T (times ``scale``) in float32.  ``tied_to`` names an Embedding whose table is the head."""
     replayable = True
 
-    def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None, scale: float = 1.0):
+    def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None, scale: float = 1.0, any_size: bool = False):
         self.vocab, self.width, self.tied_to, self.scale = vocab, width, tied_to, float(scale)
+        self.any_size = bool(any_size)   # a width that the bfloat16 product does not take goes through the plain product
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -51,14 +52,17 @@ class LMHead(Part):
         return [self.matrix()]
 
     def problems(self, dtype, page_size):
-        return needs_multiple_of_8(dtype, "width", self.width)
+        return [] if self.any_size else needs_multiple_of_8(dtype, "width", self.width)
 
     accepts_prepared = True
 
     def forward(self, ctx, rows, prepared=None):
         """``prepared``: a PreNormed whose rows these are: the product scales its result by the norm's factor."""
         logits = ctx.buffer("logits", (rows.shape[0], self.vocab), torch.float32)
-        ops.gemm(rows, self.matrix(), logits, rms_parts=prepared.as_gemm_arg() if prepared is not None else None)
+        if prepared is None and not ops.gemm_takes(rows, self.matrix()):
+            product(ctx, rows, self.matrix(), logits)
+        else:
+            ops.gemm(rows, self.matrix(), logits, rms_parts=prepared.as_gemm_arg() if prepared is not None else None)
         if self.scale != 1.0:
             ops.scale_rows(logits, self.scale)
         return logits

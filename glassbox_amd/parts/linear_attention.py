@@ -24,7 +24,7 @@ from typing import Dict, Optional, Sequence
 import torch
 
 from .. import ops
-from .base import LayerCache, Mixer, StateSpec, TensorSpec, needs_multiple_of_8, split_workspace
+from .base import LayerCache, Mixer, StateSpec, TensorSpec, product
 from .rotary import Rotary
 
 
@@ -49,7 +49,7 @@ class _LinearMixer(Mixer):
         return [self.w_in, self.wo]
 
     def problems(self, dtype, page_size):
-        out = needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "heads * vdim", self.v_dim)
+        out = []   # (sizes that the matrix-core products do not take go through the plain product)
         if self.key_dim > ops.LINEAR_MAX_KEY_DIM:
             out.append(("dim", f"{self.key_dim} is above {ops.LINEAR_MAX_KEY_DIM}, the largest key size the recurrence "
                                f"kernel takes"))
@@ -72,10 +72,10 @@ class _LinearMixer(Mixer):
         proj = ctx.buffer("lin_proj", (n, rows), ctx.dtype)
         if tail and n > ops.ROPE_PRODUCT_MAX_ROWS:
             main = rows - tail
-            ops.gemm(h, self.w_in[:main], proj[:, :main], workspace=split_workspace(ctx, n, main, self.width))
-            ops.gemm(h, self.w_in[main:], proj[:, main:], workspace=split_workspace(ctx, n, tail, self.width))
+            product(ctx, h, self.w_in[:main], proj[:, :main])
+            product(ctx, h, self.w_in[main:], proj[:, main:])
         else:
-            ops.gemm(h, self.w_in, proj, workspace=split_workspace(ctx, n, rows, self.width))
+            product(ctx, h, self.w_in, proj)
         return proj
 
     def _finish(self, ctx, proj, q32, k32, residual, cache, store, norm_weight, decay=None, head_decay=None):
@@ -94,8 +94,7 @@ class _LinearMixer(Mixer):
                         self.value_dim, decay=decay, head_decay=head_decay, segments=segments, workspace=ws)
         gated = ctx.buffer("lin_gated", (n, self.v_dim), ctx.dtype)
         ops.head_norm_gate(o, proj[:, g_off:g_off + self.v_dim], norm_weight, gated, self.n_heads, self.value_dim, self.eps)
-        ops.gemm(gated, self.wo, residual, accumulate=not store,
-                 workspace=split_workspace(ctx, n, self.width, self.v_dim))
+        product(ctx, gated, self.wo, residual, accumulate=not store)
 
 
 class Retention(_LinearMixer):
@@ -183,7 +182,7 @@ class GatedLinearAttention(_LinearMixer):
             # the second matrix of the decay's projection as a product of its own (sizes that a bfloat16 product does not
             # take: inside the kernel)
             z = ctx.buffer("lin_z", (n, self.qk_dim), torch.float32)
-            ops.gemm(proj[:, low_off:low_off + rank], self.w_a2, z)
+            product(ctx, proj[:, low_off:low_off + rank], self.w_a2, z)
         ops.gla_prep(proj, 0, self.qk_dim, low_off, self.w_a2, self.a2_bias, q32, k32, decay,
                      1.0 / math.sqrt(self.key_dim), self.tau, z=z)
         self._finish(ctx, proj, q32, k32, residual, cache, store, self.norm_weight, decay=decay)

@@ -7,15 +7,17 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, PreNormed, TensorSpec, emit_target, needs_multiple_of_8, split_workspace
+from .base import FeedForward, PreNormed, TensorSpec, emit_target, needs_multiple_of_8, product, split_workspace
 
 
 class SwiGLU(FeedForward):
     replayable = True
     taped = True
 
-    def __init__(self, width: int, intermediate: int):
-        self.width, self.intermediate = width, intermediate
+    def __init__(self, width: int, intermediate: int, any_size: bool = False):
+        """``any_size``: sizes that the bfloat16 matrix-core products do not take (no multiples of 8) are not refused but
+        go through the plain product, unfused."""
+        self.width, self.intermediate, self.any_size = width, intermediate, bool(any_size)
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -32,6 +34,8 @@ class SwiGLU(FeedForward):
         return [self.w_gate_up, self.w_down]
 
     def problems(self, dtype, page_size):
+        if self.any_size:
+            return []
         return needs_multiple_of_8(dtype, "width", self.width) + needs_multiple_of_8(dtype, "intermediate", self.intermediate)
 
     accepts_fused_norm = True
@@ -45,6 +49,13 @@ class SwiGLU(FeedForward):
         ``store``: the rows are written to ``residual`` (float32) instead of added."""
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
+        if ctx.dtype == torch.bfloat16 and (self.width % 8 or self.intermediate % 8):
+            # (only with ``any_size``, and then without norms to fuse: the blocks that offer those build it without)
+            gate_up = ctx.buffer("gate_up", (n, 2 * self.intermediate), ctx.dtype)
+            product(ctx, h, self.w_gate_up, gate_up)
+            ops.silu_mul(gate_up, act)
+            product(ctx, act, self.w_down, residual, accumulate=not store)
+            return None
         if isinstance(norm, PreNormed):
             ops.gemm(norm.rows, self.w_gate_up, act, silu_mul=True, rms_parts=norm.as_gemm_arg())
         elif ctx.dtype == torch.bfloat16 and self.intermediate % 8 == 0:

@@ -39,7 +39,7 @@ CASES: Dict[str, dict] = {
                                         "mask": {"size": 40, "keep_first": 35}}, "mlp": None},
         {"type": "gla", "mixer": {"heads": 1, "dim": 16, "vdim": 128, "tau": 16.0, "rank": 24}, "mlp": {"kind": "dense", "ff": 40}},
     ]),
-    # sizes that the bfloat16 products do not take (inner sizes that are no multiple of 8): 32-bit only
+    # sizes that the matrix-core products do not take in bfloat16 (inner sizes that are no multiple of 8): the plain product
     "O": dict(architecture="Sagalorn", vocab=53, width=50, streams=2, logit_scale=0.7, embedding={"scale": 3.0},
               norm={"eps": 1e-5}, loop={"start": 1, "stop": 2, "times": 2}, layers=[
         {"type": "retention", "mixer": {"heads": 3, "dim": 6, "vdim": 10, "decay": [0.8, 0.9, 0.99],
@@ -61,7 +61,6 @@ CASES: Dict[str, dict] = {
                                         "rot": {"dims": 16, "base": 1000.0}}, "mlp": None},
     ]),
 }
-BF16_CASES = ("P", "Q", "R", "S")
 
 
 def folder_of(base: str, name: str, seed: int = 0, std: float = 0.05) -> str:

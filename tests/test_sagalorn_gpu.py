@@ -15,7 +15,7 @@ import torch
 
 import helpers
 from plain import sagalorn as ps
-from sagalorn_cases import BF16_CASES, CASES, folder_of, rounded
+from sagalorn_cases import CASES, folder_of, rounded
 
 pytestmark = pytest.mark.gpu
 F64 = torch.float64
@@ -308,12 +308,7 @@ def _poison(engine) -> None:
 @pytest.mark.parametrize("name", list(CASES))
 def test_every_way_of_cutting_requests_into_steps(model_dirs, name, dtype):
     from glassbox_amd.engine import Engine
-    from glassbox_amd.engine.engine import EngineError
     folder = folder_of(model_dirs.base, name)
-    if dtype == "bfloat16" and name not in BF16_CASES:
-        with pytest.raises(EngineError, match="multiple of 8"):
-            Engine(folder, dtype=dtype, max_tokens=64, max_seqs=2)
-        return
     requests = _requests(CASES[name]["vocab"])
     mixed, peak = helpers.schedule_mixed(requests, seed=3, live=3, tail=20)
     eng = Engine(folder, dtype=dtype, max_tokens=max(peak, 192), max_seqs=3)
