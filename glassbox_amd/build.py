@@ -48,6 +48,8 @@ LIBRARIES: Dict[str, tuple] = {
     "sampling": ("hip", ["hip/sampling.hip"], ["hip/common.h"]),
     "streams": ("hip", ["hip/streams.hip"], ["hip/common.h"]),
     "linear_attention": ("hip", ["hip/linear_attention.hip"], ["hip/common.h"]),
+    "shortconv": ("hip", ["hip/shortconv.hip"], ["hip/common.h"]),
+    "moe": ("hip", ["hip/moe.hip"], ["hip/common.h"]),
 }
 
 _lock = threading.Lock()

@@ -2,6 +2,7 @@ from .base import (ConfigError, ModelConfig, architecture_of, config_from_dict, 
                    known_architectures, lookup, register_architecture)
 from .llama import LlamaConfig
 from .sagalorn import SagalornConfig
+from .dekinex import DekinexConfig
 
-__all__ = ["ConfigError", "ModelConfig", "LlamaConfig", "SagalornConfig", "architecture_of", "config_from_dict",
+__all__ = ["ConfigError", "ModelConfig", "LlamaConfig", "SagalornConfig", "DekinexConfig", "architecture_of", "config_from_dict",
            "config_from_dir", "known_architectures", "lookup", "register_architecture"]

@@ -832,6 +832,124 @@ extern "C" int gb_add_bias(float* x, const float* bias, int n, int d, hipStream_
   return launched("add_bias");
 }
 
+// ------------------------------------------------------------------------ embedding with a hashed pair table
+// x[c, i, :] = table[ids[i], :] + pairs[row, :], row = (previous token * mul_prev + ids[i] * mul_cur) mod buckets, and
+// row `buckets` (the table's last) for a request's first token.  The token before a step's first row of a request is
+// kept in the request's state slot (`prev`, one int32 a slot): the block of that first row reads it, unless the request
+// starts at position 0, and leaves the request's last token of this step there; no other block touches the slot.
+template <typename T>
+__global__ void embed_pairs_kernel(const T* __restrict__ table, const T* __restrict__ pairs, const int32_t* __restrict__ ids,
+                                   float* __restrict__ x, int n, int d, int vocab, int buckets, long long mul_prev,
+                                   long long mul_cur, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ q_start,
+                                   const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
+                                   const int32_t* __restrict__ state_slots, int32_t* __restrict__ prev, int copies) {
+  __shared__ int s_before;
+  const int i = blockIdx.x;
+  const int id = ids[i];
+  if (threadIdx.x == 0) {
+    const int seq = tok_seq[i], start = q_start[seq];
+    int before;
+    if (i > start) {
+      before = ids[i - 1];
+    } else {
+      int32_t* slot = prev + state_slots[seq];
+      before = pos0[seq] == 0 ? -1 : *slot;
+      *slot = ids[start + q_len[seq] - 1];
+    }
+    s_before = before;
+  }
+  __syncthreads();
+  const int before = s_before;
+  const bool ok = id >= 0 && id < vocab && before < vocab;
+  long long row = buckets;
+  if (before >= 0) {
+    row = ((long long)before * mul_prev + (long long)id * mul_cur) % buckets;
+    if (row < 0) row += buckets;
+  }
+  const T* trow = table + (size_t)(ok ? id : 0) * d;
+  const T* prow = pairs + (size_t)(ok ? row : 0) * d;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    const float v = ok ? to_f(trow[c]) + to_f(prow[c]) : __builtin_nanf("");  // a bad id must not pass silently
+    for (int k = 0; k < copies; ++k) x[((size_t)k * n + i) * d + c] = v;
+  }
+}
+
+extern "C" int gb_embed_pairs(const void* table, const void* pairs, int dtype, const int32_t* ids, float* x, int n, int d,
+                              int vocab, int buckets, long long mul_prev, long long mul_cur, const int32_t* tok_seq,
+                              const int32_t* q_start, const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots,
+                              int32_t* prev, int copies, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && d > 0 && vocab > 0 && buckets > 0 && copies > 0, "embed_pairs: bad sizes n=%d d=%d vocab=%d buckets=%d",
+             n, d, vocab, buckets);
+  GB_REQUIRE(tok_seq && q_start && q_len && pos0 && state_slots && prev, "embed_pairs: the step's tables and the state are needed");
+  if (n == 0) return 0;
+  const int threads = d >= 256 ? 256 : 64;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(embed_pairs_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)table, (const float*)pairs,
+                       ids, x, n, d, vocab, buckets, mul_prev, mul_cur, tok_seq, q_start, q_len, pos0, state_slots, prev, copies);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(embed_pairs_kernel<bf16>, dim3(n), dim3(threads), 0, stream, (const bf16*)table, (const bf16*)pairs,
+                       ids, x, n, d, vocab, buckets, mul_prev, mul_cur, tok_seq, q_start, q_len, pos0, state_slots, prev, copies);
+  else
+    return fail("embed_pairs: unknown dtype %d", dtype);
+  return launched("embed_pairs");
+}
+
+// ------------------------------------------------------------------------ gated unit with clamped halves
+// act[t, j] = g * sigmoid(alpha * g) * (u + 1), g = min(gate[t, j], limit), u = clamp(up[t, j], -limit, limit); the rows of
+// `gu` hold the gate columns, then the up columns (of the product's 32-bit sums or of the activations' type).
+template <typename I, typename O>
+__global__ void glu_clamped_kernel(const I* __restrict__ gu, int ld, O* __restrict__ act, long long count, int inter,
+                                   float limit, float alpha) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  const long long t = idx / inter;
+  const int j = (int)(idx % inter);
+  const I* row = gu + (size_t)t * ld;
+  const float g = fminf(to_f(row[j]), limit);
+  const float u = fminf(fmaxf(to_f(row[inter + j]), -limit), limit);
+  act[idx] = from_f<O>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+}
+
+extern "C" int gb_glu_clamped(const void* gu, int in_dtype, int ld, void* act, int out_dtype, int n, int inter, float limit,
+                              float alpha, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && inter > 0 && ld >= 2 * inter, "glu_clamped: bad sizes n=%d inter=%d ld=%d", n, inter, ld);
+  if (n == 0) return 0;
+  const long long count = (long long)n * inter;
+  GB_REQUIRE((count + 255) / 256 < (1ll << 31), "glu_clamped: too many elements");
+  const dim3 grid((unsigned)((count + 255) / 256));
+  if (in_dtype == kF32 && out_dtype == kF32)
+    hipLaunchKernelGGL((glu_clamped_kernel<float, float>), grid, dim3(256), 0, stream, (const float*)gu, ld, (float*)act, count, inter, limit, alpha);
+  else if (in_dtype == kF32 && out_dtype == kBF16)
+    hipLaunchKernelGGL((glu_clamped_kernel<float, bf16>), grid, dim3(256), 0, stream, (const float*)gu, ld, (bf16*)act, count, inter, limit, alpha);
+  else if (in_dtype == kBF16 && out_dtype == kBF16)
+    hipLaunchKernelGGL((glu_clamped_kernel<bf16, bf16>), grid, dim3(256), 0, stream, (const bf16*)gu, ld, (bf16*)act, count, inter, limit, alpha);
+  else
+    return fail("glu_clamped: no kernel for operand type %d and result type %d", in_dtype, out_dtype);
+  return launched("glu_clamped");
+}
+
+// ------------------------------------------------------------------------ scaled add
+// x[r, c] += alpha * y[r, c] + bias[c]   (float32; y or bias may be absent): a residual that takes its layer's sum times
+// a constant, or another residual and a vector
+__global__ void axpy_rows_kernel(float* __restrict__ x, const float* __restrict__ y, float alpha, const float* __restrict__ bias,
+                                 long long count, int d) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  float v = x[idx];
+  if (y) v = fmaf(alpha, y[idx], v);
+  if (bias) v += bias[idx % d];
+  x[idx] = v;
+}
+
+extern "C" int gb_axpy_rows(float* x, const float* y, float alpha, const float* bias, int n, int d, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && d > 0, "axpy_rows: bad sizes n=%d d=%d", n, d);
+  if (n == 0) return 0;
+  const long long count = (long long)n * d;
+  GB_REQUIRE((count + 255) / 256 < (1ll << 31), "axpy_rows: too many elements");
+  hipLaunchKernelGGL(axpy_rows_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, x, y, alpha, bias, count, d);
+  return launched("axpy_rows");
+}
+
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_embed)
 GB_TAPED(gb_rmsnorm)
@@ -843,3 +961,5 @@ GB_TAPED(gb_qk_norm_store)
 GB_TAPED(gb_add_bias)
 GB_TAPED(gb_scale_rows)
 GB_TAPED(gb_gemm_plain)
+GB_TAPED(gb_glu_clamped)
+GB_TAPED(gb_axpy_rows)

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ a, const float* __restrict__ head_decay,
     const T* __restrict__ v, int v_stride, float* __restrict__ out, float* __restrict__ state,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
-    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int segs, int seg_len, float* __restrict__ seg_state,
+    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int sc, int a_head, int segs, int seg_len, float* __restrict__ seg_state,
     float* __restrict__ seg_decay) {
   constexpr int DKP = R * kLanesCol;                       // rows, padded
   constexpr int PER = (kTokens * DKP) / kThreads;          // staged elements a thread and array (R >= 2)
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(
   const bool cut = sg.n_segs > 1;                           // the request's portion runs as several segments
 
   float S[R], P[GATED ? R : 1];
-  float* slot_row = state + (((size_t)state_slots[seq] * nh + h) * dv + (live ? col : 0)) * dk + rg * R;
+  float* slot_row = state + (((size_t)state_slots[seq] * nh + h) * sc + (live ? col : 0)) * dk + rg * R;
   // where the end state goes: the request's slot, or, of a segment, the workspace
   float* srow = cut ? seg_state + (((size_t)blockIdx.z * nh + h) * dv + (live ? col : 0)) * dk + rg * R : slot_row;
   // a request's first tokens start from an empty state, whatever the slot held; so does every segment but the first
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(
       const size_t at = (size_t)(first + t0 + tok) * width + (size_t)h * dk + ch;
       nq[e] = ok ? q[at] : 0.f;
       nk[e] = ok ? k[at] : 0.f;
-      if (GATED) na[e] = ok ? a[at] : 0.f;
+      if (GATED) na[e] = ok ? a[a_head ? (size_t)(first + t0 + tok) * nh + h : at] : 0.f;
     }
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
@@ -201,7 +201,7 @@ template <int R, bool GATED>
 __global__ __launch_bounds__(kThreads) void scan_join_kernel(
     const float* __restrict__ q, const float* __restrict__ a, const float* __restrict__ head_decay, float* __restrict__ out,
     float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
-    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int segs, int seg_len, const float* __restrict__ seg_state,
+    const int32_t* __restrict__ state_slots, int nh, int dk, int dv, int sc, int a_head, int segs, int seg_len, const float* __restrict__ seg_state,
     const float* __restrict__ seg_decay) {
   constexpr int DKP = R * kLanesCol;
   constexpr int PER = (kTokens * DKP) / kThreads;
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void scan_join_kernel(
       const bool ok = t0 + tok < count && ch < dk;
       const size_t at = (size_t)(first + t0 + tok) * width + (size_t)h * dk + ch;
       nq[e] = ok ? q[at] : 0.f;
-      if (GATED) na[e] = ok ? a[at] : 0.f;
+      if (GATED) na[e] = ok ? a[a_head ? (size_t)(first + t0 + tok) * nh + h : at] : 0.f;
     }
   };
   fetch(0);
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(kThreads) void scan_join_kernel(
   }
   if (sg.seg == sg.n_segs - 1 && live) {   // the request's state after the portion
     const float* e = e_row(sg.seg);
-    float* srow = state + (((size_t)state_slots[sg.seq] * nh + h) * dv + col) * dk + rg * R;
+    float* srow = state + (((size_t)state_slots[sg.seq] * nh + h) * sc + col) * dk + rg * R;
 #pragma unroll
     for (int m = 0; m < R; ++m)
       if (rg * R + m < dk) srow[m] = fmaf(P[m], S0[m], e[m]);
@@ -454,18 +454,120 @@ __global__ __launch_bounds__(256) void head_norm_gate_words_kernel(const float* 
   }
 }
 
+// ---------------------------------------------------------------- matrix memory with exponential gates (mLSTM)
+// Per head, with a log input gate i_t, a log forget gate f_t and a running maximum m (m before the first token: 0):
+//   m_t = max(f_t + m_(t-1), i_t)
+//   S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t the same with k_t alone
+//   o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+// which is the recurrence above with the decay a_t = exp(f_t + m_(t-1) - m_t) a token and head, the keys times
+// b_t = exp(i_t - m_t), and n as one more value channel whose v is 1.  The gates are capped,
+// i = cap tanh(z_i / cap), f = log sigmoid(cap tanh(z_f / cap)), z the projections plus their biases.
+
+// One wave a (request, head): 64 tokens at a time, each lane its token's gates; m over the 64 by a scan of the pairs
+// (F, I) that stand for m -> max(F + m, I) (first (F1, I1), then (F2, I2): (F1 + F2, max(I1 + F2, I2))).  Writes
+// coef[t, h] = (a_t, b_t, exp(-m_t)) and leaves the request's last m in its state slot at `m_at` of the head's block.
+__global__ __launch_bounds__(kWave) void mlstm_gates_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ bias_i,
+                                                          const float* __restrict__ bias_f, float cap, float* __restrict__ coef,
+                                                          float* __restrict__ state, long long head_floats, long long m_at,
+                                                          const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                                                          const int32_t* __restrict__ pos0, const int32_t* __restrict__ state_slots,
+                                                          int nh) {
+  const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int start = q_start[seq], L = q_len[seq];
+  float* mp = state + ((size_t)state_slots[seq] * nh + h) * head_floats + m_at;
+  float carry = pos0[seq] == 0 ? 0.f : *mp;
+  const float bi = bias_i ? bias_i[h] : 0.f, bf = bias_f ? bias_f[h] : 0.f;
+  for (int base = 0; base < L; base += kWave) {
+    const int t = base + lane;
+    const bool valid = t < L;
+    float ig = -INFINITY, fg = 0.f;
+    if (valid) {
+      const float* row = z + (size_t)(start + t) * ldz;
+      ig = cap * tanhf((row[h] + bi) / cap);
+      fg = log_sigmoid(cap * tanhf((row[nh + h] + bf) / cap));
+    }
+    float F = fg, I = ig;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const float Fo = __shfl_up(F, off, kWave), Io = __shfl_up(I, off, kWave);
+      if (lane >= off) {
+        I = fmaxf(Io + F, I);
+        F = Fo + F;
+      }
+    }
+    const float m = fmaxf(F + carry, I);
+    float before = __shfl_up(m, 1, kWave);
+    if (lane == 0) before = carry;
+    if (valid) {
+      float* c = coef + ((size_t)(start + t) * nh + h) * 3;
+      c[0] = expf(fg + before - m);
+      c[1] = expf(ig - m);
+      c[2] = expf(-m);
+    }
+    carry = __shfl(m, kWave - 1, kWave);   // (lanes beyond the last token hold the identity: their m is the last token's)
+  }
+  if (lane == 0 && L > 0) *mp = carry;
+}
+
+// q32 = q * q_scale, k32 = k * b_t, decay[t, h] = a_t, vext[t, h, :] = (v[t, h, :], 1): the scan's operands
+template <typename T>
+__global__ void mlstm_prep_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off,
+                                  const float* __restrict__ coef, float* __restrict__ q32, float* __restrict__ k32,
+                                  float* __restrict__ decay, T* __restrict__ vext, int nh, int dk, int dv, float q_scale) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * stride;
+  const int width = nh * dk, vw = nh * (dv + 1);
+  for (int c = blockIdx.y * kPiece + threadIdx.x; c < min(width, (int)(blockIdx.y + 1) * kPiece); c += blockDim.x) {
+    const int h = c / dk;
+    q32[(size_t)t * width + c] = to_f(row[q_off + c]) * q_scale;
+    k32[(size_t)t * width + c] = to_f(row[k_off + c]) * coef[((size_t)t * nh + h) * 3 + 1];
+  }
+  for (int c = blockIdx.y * kPiece + threadIdx.x; c < min(vw, (int)(blockIdx.y + 1) * kPiece); c += blockDim.x) {
+    const int h = c / (dv + 1), d = c % (dv + 1);
+    vext[(size_t)t * vw + c] = d < dv ? row[v_off + h * dv + d] : from_f<T>(1.0f);
+  }
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < nh; h += blockDim.x) decay[(size_t)t * nh + h] = coef[((size_t)t * nh + h) * 3];
+}
+
+// out[t, h, :] = w[h, :] * y / sqrt(mean(y^2) + eps) * sigmoid(gate[t, h, :]),  y = o[t, h, :dv] / (max(|o[t, h, dv]|,
+// exp(-m_t)) + 1e-6); o holds dv + 1 sums a head, the last the normaliser's.  One wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(4 * kWave) void mlstm_out_kernel(const float* __restrict__ o, const float* __restrict__ coef,
+                                                            const T* __restrict__ gate, int gate_stride,
+                                                            const float* __restrict__ w, T* __restrict__ out, int nh, int dv,
+                                                            float eps, int pairs) {
+  const int pair = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (pair >= pairs) return;
+  const int t = pair / nh, h = pair % nh, lane = threadIdx.x % kWave;
+  const float* orow = o + ((size_t)t * nh + h) * (dv + 1);
+  const float den = fmaxf(fabsf(orow[dv]), coef[((size_t)t * nh + h) * 3 + 2]) + 1e-6f;
+  float ss = 0.f;
+  for (int d = lane; d < dv; d += kWave) {
+    const float y = orow[d] / den;
+    ss = fmaf(y, y, ss);
+  }
+  ss = wave_sum(ss);
+  const float s = 1.0f / sqrtf(ss / (float)dv + eps);
+  for (int d = lane; d < dv; d += kWave) {
+    const float g = to_f(gate[(size_t)t * gate_stride + (size_t)h * dv + d]);
+    const float y = (w ? w[(size_t)h * dv + d] : 1.0f) * ((orow[d] / den) * s);
+    out[((size_t)t * nh + h) * dv + d] = from_f<T>(y / (1.0f + expf(-g)));
+  }
+}
+
 template <typename T, bool GATED>
 int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const float* k, const float* a, const float* head_decay,
                 const void* v, int v_stride, float* out, float* state, const int32_t* q_start, const int32_t* q_len,
-                const int32_t* pos0, const int32_t* slots, int nh, int dk, int dv, int segs, int seg_len, float* seg_state,
+                const int32_t* pos0, const int32_t* slots, int nh, int dk, int dv, int sc, int a_head, int segs, int seg_len, float* seg_state,
                 float* seg_decay) {
 #define GB_SCAN(RR)                                                                                                          \
   case RR:                                                                                                                   \
     hipLaunchKernelGGL((scan_kernel<T, RR, GATED>), grid, dim3(kThreads), 0, stream, q, k, a, head_decay, (const T*)v, v_stride, \
-                       out, state, q_start, q_len, pos0, slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);            \
+                       out, state, q_start, q_len, pos0, slots, nh, dk, dv, sc, a_head, segs, seg_len, seg_state, seg_decay); \
     if (segs > 1)                                                                                                            \
       hipLaunchKernelGGL((scan_join_kernel<RR, GATED>), grid, dim3(kThreads), 0, stream, q, a, head_decay, out, state, q_start, \
-                         q_len, slots, nh, dk, dv, segs, seg_len, (const float*)seg_state, (const float*)seg_decay);         \
+                         q_len, slots, nh, dk, dv, sc, a_head, segs, seg_len, (const float*)seg_state, (const float*)seg_decay); \
     break;
   switch (R) {
     GB_SCAN(2) GB_SCAN(4) GB_SCAN(8) GB_SCAN(16) GB_SCAN(32)
@@ -477,9 +579,10 @@ int launch_scan(int R, dim3 grid, hipStream_t stream, const float* q, const floa
 
 }  // namespace
 
-// The recurrence over the rows of a step.  q, k [n, nh * dk] float32; `a` [n, nh * dk] float32 decays a key channel, or
+// The recurrence over the rows of a step.  q, k [n, nh * dk] float32; `a` [n, nh * dk] float32 decays a key channel
+// (a_head: [n, nh], a decay a token and head, the same for all its key channels), or
 // nullptr with head_decay [nh] float32; v rows of nh * dv in the activations' type (row stride v_stride); out [n, nh * dv]
-// float32; state [slots, nh, dv, dk] float32.  Request s of the step brings rows q_start[s] .. + q_len[s] - 1, starts at
+// float32; state [slots, nh, state_cols, dk] float32 with state_cols >= dv (rows beyond dv are the caller's).  Request s of the step brings rows q_start[s] .. + q_len[s] - 1, starts at
 // position pos0[s] (0: from an empty state) and keeps its state in slot state_slots[s].
 // segs > 1: no request brings more than segs * seg_len rows, and those that bring more than seg_len run as segments of
 // seg_len rows side by side; seg_ws holds gb_linear_scan_floats(n_seqs, nh, dk, dv, segs) floats.
@@ -490,8 +593,9 @@ extern "C" long long gb_linear_scan_floats(int n_seqs, int nh, int dk, int dv, i
 extern "C" int gb_linear_scan(const float* q, const float* k, const float* a, const float* head_decay, const void* v,
                               int v_dtype, int v_stride, float* out, float* state, const int32_t* q_start,
                               const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
-                              int dk, int dv, int segs, int seg_len, float* seg_ws, long long seg_ws_floats,
+                              int dk, int dv, int state_cols, int a_head, int segs, int seg_len, float* seg_ws, long long seg_ws_floats,
                               hipStream_t stream) {
+  GB_REQUIRE(state_cols >= dv, "linear_scan: a state of %d columns a head holds fewer than the %d value channels", state_cols, dv);
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes requests=%d heads=%d dk=%d dv=%d", n_seqs, nh, dk, dv);
   GB_REQUIRE(dk <= 32 * kLanesCol, "linear_scan: a key size of %d is above the supported %d", dk, 32 * kLanesCol);
   GB_REQUIRE((a != nullptr) != (head_decay != nullptr), "linear_scan: a decay a head or a decay a key channel, one of the two");
@@ -509,11 +613,11 @@ extern "C" int gb_linear_scan(const float* q, const float* k, const float* a, co
   const dim3 grid((unsigned)((dv + kColsBlock - 1) / kColsBlock), (unsigned)nh, (unsigned)(n_seqs * segs));
   const bool gated = a != nullptr;
   if (v_dtype == kF32)
-    return gated ? launch_scan<float, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay)
-                 : launch_scan<float, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);
+    return gated ? launch_scan<float, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, state_cols, a_head, segs, seg_len, seg_state, seg_decay)
+                 : launch_scan<float, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, state_cols, a_head, segs, seg_len, seg_state, seg_decay);
   if (v_dtype == kBF16)
-    return gated ? launch_scan<bf16, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay)
-                 : launch_scan<bf16, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, segs, seg_len, seg_state, seg_decay);
+    return gated ? launch_scan<bf16, true>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, state_cols, a_head, segs, seg_len, seg_state, seg_decay)
+                 : launch_scan<bf16, false>(R, grid, stream, q, k, a, head_decay, v, v_stride, out, state, q_start, q_len, pos0, state_slots, nh, dk, dv, state_cols, a_head, segs, seg_len, seg_state, seg_decay);
   return fail("linear_scan: unknown dtype %d", v_dtype);
 }
 
@@ -587,7 +691,65 @@ extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, in
   return launched("head_norm_gate");
 }
 
+// z [n, ldz] float32: the input gates' projections of the nh heads, then the forget gates'; biases float32 [nh] or nullptr;
+// coef [n, nh, 3] float32 receives (a_t, b_t, exp(-m_t)); the running maximum of head h of a request lives at
+// state[slot][h * head_floats + m_at].
+extern "C" int gb_mlstm_gates(const float* z, int ldz, const float* bias_i, const float* bias_f, float cap, float* coef,
+                              float* state, long long head_floats, long long m_at, const int32_t* q_start,
+                              const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
+                              hipStream_t stream) {
+  GB_REQUIRE(n_seqs >= 0 && nh > 0 && ldz >= 2 * nh && cap > 0.f, "mlstm_gates: bad sizes requests=%d heads=%d ldz=%d cap=%g", n_seqs, nh, ldz, cap);
+  GB_REQUIRE(head_floats > 0 && m_at >= 0 && m_at < head_floats, "mlstm_gates: the maximum lies outside its head's state");
+  GB_REQUIRE(n_seqs <= 2147483647 && nh <= 65535, "mlstm_gates: too many heads for one launch");
+  if (n_seqs == 0) return 0;
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(n_seqs, nh), dim3(kWave), 0, stream, z, ldz, bias_i, bias_f, cap, coef, state,
+                     head_floats, m_at, q_start, q_len, pos0, state_slots, nh);
+  return launched("mlstm_gates");
+}
+
+extern "C" int gb_mlstm_prep(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off, const float* coef,
+                             float* q32, float* k32, float* decay, void* vext, int n, int nh, int dk, int dv, float q_scale,
+                             hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh > 0 && dk > 0 && dv > 0, "mlstm_prep: bad sizes n=%d heads=%d dk=%d dv=%d", n, nh, dk, dv);
+  GB_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + nh * dk <= stride && k_off + nh * dk <= stride &&
+                 v_off + nh * dv <= stride, "mlstm_prep: heads beyond the row");
+  const int longest = nh * dk > nh * (dv + 1) ? nh * dk : nh * (dv + 1);
+  GB_REQUIRE((longest + kPiece - 1) / kPiece <= 65535, "mlstm_prep: rows too long for one launch");
+  if (n == 0) return 0;
+  const dim3 grid(n, (longest + kPiece - 1) / kPiece);
+  const int threads = longest >= 512 ? 256 : 128;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(mlstm_prep_kernel<float>, grid, dim3(threads), 0, stream, (const float*)proj, stride, q_off, k_off, v_off, coef,
+                       q32, k32, decay, (float*)vext, nh, dk, dv, q_scale);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(mlstm_prep_kernel<bf16>, grid, dim3(threads), 0, stream, (const bf16*)proj, stride, q_off, k_off, v_off, coef,
+                       q32, k32, decay, (bf16*)vext, nh, dk, dv, q_scale);
+  else
+    return fail("mlstm_prep: unknown dtype %d", dtype);
+  return launched("mlstm_prep");
+}
+
+extern "C" int gb_mlstm_out(const float* o, const float* coef, const void* gate, int dtype, int gate_stride, const float* w,
+                            void* out, int n, int nh, int dv, float eps, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && nh > 0 && dv > 0 && gate_stride >= nh * dv, "mlstm_out: bad sizes n=%d heads=%d dv=%d", n, nh, dv);
+  GB_REQUIRE((long long)n * nh < (1ll << 31), "mlstm_out: too many (token, head) pairs");
+  if (n == 0) return 0;
+  const dim3 grid((unsigned)((n * nh + 3) / 4));
+  if (dtype == kF32)
+    hipLaunchKernelGGL(mlstm_out_kernel<float>, grid, dim3(4 * kWave), 0, stream, o, coef, (const float*)gate, gate_stride, w,
+                       (float*)out, nh, dv, eps, n * nh);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(mlstm_out_kernel<bf16>, grid, dim3(4 * kWave), 0, stream, o, coef, (const bf16*)gate, gate_stride, w,
+                       (bf16*)out, nh, dv, eps, n * nh);
+  else
+    return fail("mlstm_out: unknown dtype %d", dtype);
+  return launched("mlstm_out");
+}
+
 GB_TAPED(gb_linear_scan)
 GB_TAPED(gb_retention_prep)
 GB_TAPED(gb_gla_prep)
 GB_TAPED(gb_head_norm_gate)
+GB_TAPED(gb_mlstm_gates)
+GB_TAPED(gb_mlstm_prep)
+GB_TAPED(gb_mlstm_out)

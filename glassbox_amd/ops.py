@@ -54,6 +54,28 @@ _SIGS = {
         "gb_scale_rows": [_vp, _f, C.c_longlong, _vp],
         # a, lda, w, ldw, c, ldc, operand dtype, result dtype, M, N, K, accumulate, stream
         "gb_gemm_plain": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+        # table, pairs, dtype, ids, x, n, d, vocab, buckets, mul_prev, mul_cur, tok_seq, q_start, q_len, pos0, state slots,
+        # prev, copies, stream
+        "gb_embed_pairs": [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _vp, _vp,
+                           _i, _vp],
+        # gate_up, its dtype, ld, act, its dtype, n, inter, limit, alpha, stream
+        "gb_glu_clamped": [_vp, _i, _i, _vp, _i, _i, _i, _f, _f, _vp],
+        # x, y, alpha, bias, n, d, stream
+        "gb_axpy_rows": [_vp, _vp, _f, _vp, _i, _i, _vp],
+    },
+    "shortconv": {
+        # proj, dtype, stride, wconv, taps, state, tok_seq, q_start, pos0, state slots, cos, sin, rot, eps, norm, out,
+        # out stride, hd, slots, k, v, page, n, nh, nkv, dim, vdim, update_state, stream
+        "gb_conv_heads": [_vp, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp, _i, _i, _vp, _vp, _vp, _i,
+                          _i, _i, _i, _i, _i, _i, _vp],
+        # proj, dtype, stride, state, q_start, q_len, state slots, requests, channels, taps, stream
+        "gb_conv_state": [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    },
+    "moe": {
+        # z, ldz, n, experts, correction, top, scale, shared, combine, ids, weights, stream
+        "gb_moe_route": [_vp, _i, _i, _i, _vp, _i, _f, _i, _vp, _vp, _vp, _vp],
+        # gate_up, its dtype, ld, combine, its columns, act, its dtype, n, inter, experts, ff, stream
+        "gb_moe_gated_units": [_vp, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     },
     "streams": {
         # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, mix, w_out, y, stream
@@ -62,9 +84,16 @@ _SIGS = {
     },
     "linear_attention": {
         # q, k, decays, head decays, v, v dtype, v stride, out, state, q_start, q_len, pos0, state slots, requests, heads,
-        # dk, dv, segments, rows a segment, workspace, its floats, stream
-        "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp,
+        # dk, dv, state columns a head, decay a head (0/1), segments, rows a segment, workspace, its floats, stream
+        "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                            C.c_longlong, _vp],
+        # z, ldz, bias_i, bias_f, cap, coef, state, floats a head, where m lies, q_start, q_len, pos0, state slots,
+        # requests, heads, stream
+        "gb_mlstm_gates": [_vp, _i, _vp, _vp, _f, _vp, _vp, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _i, _i, _vp],
+        # proj, dtype, stride, q_off, k_off, v_off, coef, q32, k32, decay, vext, n, heads, dk, dv, q_scale, stream
+        "gb_mlstm_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
+        # o, coef, gate, dtype, gate stride, w, out, n, heads, dv, eps, stream
+        "gb_mlstm_out": [_vp, _vp, _vp, _i, _i, _vp, _vp, _i, _i, _i, _f, _vp],
         # proj, dtype, stride, q_off, k_off, cos, sin, q32, k32, n, heads, dk, rot, k_scale, stream
         "gb_retention_prep": [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
         # proj, dtype, stride, q_off, k_off, low_off, a2, z, a2 bias, q32, k32, decay, n, width, rank, q_scale, 1/tau, stream
@@ -642,7 +671,7 @@ def linear_scan_segments(max_q_len: int) -> int:
 def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torch.Tensor, state: torch.Tensor, ctx,
                 n_heads: int, key_dim: int, value_dim: int, decay: Optional[torch.Tensor] = None,
                 head_decay: Optional[torch.Tensor] = None, segments: int = 1,
-                workspace: Optional[torch.Tensor] = None) -> None:
+                workspace: Optional[torch.Tensor] = None, token_decay: Optional[torch.Tensor] = None) -> None:
     """The recurrence S <- diag(a) S + k v^T, o = S^T q over each request's rows of the step, in their order, from the
     state in the request's slot (empty for a request at position 0) and back into it.  ``decay`` float32
     [n, heads * key_dim] (a decay a key channel and token) or ``head_decay`` float32 [heads]; ``v`` rows of
@@ -650,22 +679,33 @@ def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torc
     ``state`` float32 [slots, heads, value_dim, key_dim].  ``segments`` > 1 (``linear_scan_segments`` of the step's
     longest portion, with a float32 ``workspace`` of requests * segments * heads * (value_dim + 1) * key_dim elements): long
     portions run as segments of ``LINEAR_SEGMENT`` rows side by side and a second kernel joins them; what a token gets then
-    differs from the token-by-token sums by rounding."""
-    _dev(q32, k32, v, out, state, decay, head_decay)
+    differs from the token-by-token sums by rounding.  ``token_decay`` float32 [n, heads], in place of the other two: a
+    decay a token and head, the same for all key channels.  ``state`` may hold more than value_dim columns a head
+    ([slots, heads, columns, key_dim]): the recurrence keeps the first value_dim, the rest are the caller's."""
+    _dev(q32, k32, v, out, state, decay, head_decay, token_decay)
+    a_head = token_decay is not None
+    if a_head:
+        if decay is not None or head_decay is not None:
+            raise KernelError("linear_scan: a decay a head, a key channel, or a token and head: one of the three")
+        _f32_rows(token_decay, (q32.shape[0], n_heads), "token_decay")
+        decay = token_decay
     n = q32.shape[0]
     _f32_rows(q32, (n, n_heads * key_dim), "q32")
     _f32_rows(k32, (n, n_heads * key_dim), "k32")
     _f32_rows(out, (n, n_heads * value_dim), "out")
     if (decay is None) == (head_decay is None):
         raise KernelError("linear_scan: a decay a head or a decay a key channel, one of the two")
-    if decay is not None:
+    if a_head:
+        pass
+    elif decay is not None:
         _f32_rows(decay, (n, n_heads * key_dim), "decay")
     else:
         _f32_rows(head_decay, (n_heads,), "head_decay")
     if v.shape != (n, n_heads * value_dim):
         raise KernelError("linear_scan: v must be [n, heads * value_dim]")
-    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, value_dim, key_dim):
-        raise KernelError("linear_scan: state must be contiguous float32 [slots, heads, value_dim, key_dim]")
+    if (state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1] != n_heads
+            or state.shape[2] < value_dim or state.shape[3] != key_dim):
+        raise KernelError("linear_scan: state must be contiguous float32 [slots, heads, value_dim or more, key_dim]")
     if key_dim > LINEAR_MAX_KEY_DIM:
         raise KernelError(f"linear_scan: a key size of {key_dim} is above {LINEAR_MAX_KEY_DIM}")
     if segments > 1:
@@ -676,7 +716,7 @@ def linear_scan(q32: torch.Tensor, k32: torch.Tensor, v: torch.Tensor, out: torc
     lib = _lib("linear_attention")
     _launch(lib, lib.gb_linear_scan, _p(q32), _p(k32), _p(decay), _p(head_decay), _p(v), dtype_code(v), _rows(v, "v"), _p(out),
             _p(state), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0), _p(ctx.state_slots), ctx.num_seqs, n_heads, key_dim,
-            value_dim, int(segments), LINEAR_SEGMENT, _p(workspace) if segments > 1 else None,
+            value_dim, int(state.shape[2]), 1 if a_head else 0, int(segments), LINEAR_SEGMENT, _p(workspace) if segments > 1 else None,
             workspace.numel() if segments > 1 else 0, _stream())
 
 
@@ -695,6 +735,213 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.T
     lib = _lib("linear_attention")
     _launch(lib, lib.gb_head_norm_gate, _p(o), _p(gate), dtype_code(out), _rows(gate, "gate"), _p(weight), _p(out), n, n_heads,
             value_dim, float(eps), _stream())
+
+
+# ------------------------------------------------------------------- matrix memory with exponential gates
+def mlstm_gates(z: torch.Tensor, bias_i: Optional[torch.Tensor], bias_f: Optional[torch.Tensor], cap: float,
+                coef: torch.Tensor, state: torch.Tensor, m_row: int, ctx, n_heads: int) -> None:
+    """coef[t, h] = (a, b, exp(-m)) float32 [n, heads, 3] from the gates' projections ``z`` float32 [n, 2 * heads] (input
+    gates, then forget gates) and their biases (float32 [heads]): i = cap tanh(z_i / cap), f = log sigmoid(cap tanh(z_f /
+    cap)), m_t = max(f_t + m_(t-1), i_t), a = exp(f + m_(t-1) - m), b = exp(i - m), over each request's rows in their
+    order.  m before a request's first token is 0; between steps it lives in element 0 of row ``m_row`` of the head's
+    block of ``state`` ([slots, heads, rows, key size] float32)."""
+    _dev(z, bias_i, bias_f, coef, state)
+    n = z.shape[0]
+    if z.dtype != torch.float32 or z.dim() != 2 or z.stride(1) != 1 or z.shape[1] < 2 * n_heads:
+        raise KernelError("mlstm_gates: z must be float32 [n, 2 * heads] with dense rows")
+    _f32_rows(coef, (n, n_heads, 3), "coef")
+    for b in (bias_i, bias_f):
+        if b is not None:
+            _f32_rows(b, (n_heads,), "gate bias")
+    if (state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1] != n_heads
+            or not 0 <= m_row < state.shape[2]):
+        raise KernelError("mlstm_gates: state must be contiguous float32 [slots, heads, rows, key size] and hold the row of m")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_mlstm_gates, _p(z), z.stride(0), _p(bias_i), _p(bias_f), float(cap), _p(coef), _p(state),
+            int(state.shape[2] * state.shape[3]), int(m_row * state.shape[3]), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0),
+            _p(ctx.state_slots), ctx.num_seqs, n_heads, _stream())
+
+
+def mlstm_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, coef: torch.Tensor, q32: torch.Tensor,
+               k32: torch.Tensor, decay: torch.Tensor, vext: torch.Tensor, n_heads: int, key_dim: int, value_dim: int,
+               q_scale: float) -> None:
+    """The recurrence's operands from the projection's rows and ``mlstm_gates``' coefficients: q32 = q * q_scale,
+    k32 = k * b (float32 [n, heads * key_dim]), decay = a (float32 [n, heads]), vext = (v, 1) a head
+    ([n, heads * (value_dim + 1)] in the projection's type: the normaliser is one more value channel)."""
+    _dev(proj, coef, q32, k32, decay, vext)
+    n = proj.shape[0]
+    stride = _rows(proj, "proj")
+    _f32_rows(coef, (n, n_heads, 3), "coef")
+    _f32_rows(q32, (n, n_heads * key_dim), "q32")
+    _f32_rows(k32, (n, n_heads * key_dim), "k32")
+    _f32_rows(decay, (n, n_heads), "decay")
+    if vext.shape != (n, n_heads * (value_dim + 1)) or vext.dtype != proj.dtype or not vext.is_contiguous():
+        raise KernelError("mlstm_prep: vext must be contiguous [n, heads * (value_dim + 1)] of the projection's type")
+    if max(q_off, k_off) + n_heads * key_dim > proj.shape[1] or v_off + n_heads * value_dim > proj.shape[1]:
+        raise KernelError("mlstm_prep: the heads lie beyond the projection's rows")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_mlstm_prep, _p(proj), dtype_code(proj), stride, int(q_off), int(k_off), int(v_off), _p(coef), _p(q32),
+            _p(k32), _p(decay), _p(vext), n, n_heads, key_dim, value_dim, float(q_scale), _stream())
+
+
+def mlstm_out(o: torch.Tensor, coef: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor,
+              n_heads: int, value_dim: int, eps: float) -> None:
+    """out[t, h] = weight[h] * y / sqrt(mean(y^2) + eps) * sigmoid(gate[t, h]) with y = o[t, h, :value_dim] /
+    (max(|o[t, h, value_dim]|, exp(-m)) + 1e-6): ``o`` float32 [n, heads * (value_dim + 1)] as the recurrence leaves it
+    (the last sum of a head is the normaliser's), ``weight`` float32 [heads * value_dim] or None, gate and out in the
+    activations' type."""
+    _dev(o, coef, gate, weight, out)
+    n = o.shape[0]
+    _f32_rows(o, (n, n_heads * (value_dim + 1)), "o")
+    _f32_rows(coef, (n, n_heads, 3), "coef")
+    if gate.shape != (n, n_heads * value_dim) or out.shape != (n, n_heads * value_dim) or gate.dtype != out.dtype \
+            or not out.is_contiguous():
+        raise KernelError("mlstm_out: gate and out must be [n, heads * value_dim] of one type, out contiguous")
+    if weight is not None:
+        _f32_rows(weight, (n_heads * value_dim,), "weight")
+    lib = _lib("linear_attention")
+    _launch(lib, lib.gb_mlstm_out, _p(o), _p(coef), _p(gate), dtype_code(out), _rows(gate, "gate"), _p(weight), _p(out), n,
+            n_heads, value_dim, float(eps), _stream())
+
+
+# ------------------------------------------------------------------- short convolution before attention
+CONV_MAX_TAPS = 8   # shortconv.hip keeps a channel's slot in registers
+
+
+def conv_heads(proj: torch.Tensor, wconv: Optional[torch.Tensor], state: Optional[torch.Tensor], ctx,
+               cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot: int, eps: float, norm: bool, out: torch.Tensor,
+               head_cols: int, slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+               n_heads: int, n_kv_heads: int, dim: int, vdim: int) -> None:
+    """The heads of a step's stacked projections made ready for attention.  ``proj`` [n, heads * dim + kv heads * (dim +
+    vdim)]: query heads, key heads, value heads.  ``wconv`` float32 [channels, taps] (None: no convolution): every
+    channel is convolved over its request's tokens, y_t = sum_j w[:, j] u_(t - taps + 1 + j), zeros before the first
+    token; the last taps - 1 projections of each request live in ``state`` (float32 [slots, taps - 1, channels]) and are
+    moved on by this call.  Then the first ``rot`` channels of every query and key head are turned in neighbouring pairs
+    by the rows' angles (``cos``, ``sin`` float32 [n, rot / 2]) and, with ``norm``, every query and key head is divided
+    by its root mean square.  ``out`` [n, (heads + 2 kv heads) * head_cols] receives the heads, each filled up with
+    zeros to ``head_cols`` columns; with ``slots`` keys and values also go to the pages (heads of ``head_cols``)."""
+    _dev(proj, wconv, state, cos, sin, out, slots, k_pages, v_pages)
+    n = proj.shape[0]
+    channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
+    taps = 1
+    if wconv is not None:
+        taps = wconv.shape[1]
+        _f32_rows(wconv, (channels, taps), "wconv")
+        if taps > CONV_MAX_TAPS:
+            raise KernelError(f"conv_heads: {taps} taps are above {CONV_MAX_TAPS}")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                         or tuple(state.shape[1:]) != (taps - 1, channels)):
+            raise KernelError("conv_heads: state must be contiguous float32 [slots, taps - 1, channels]")
+    if proj.shape[1] < channels or out.shape != (n, (n_heads + 2 * n_kv_heads) * head_cols) or out.dtype != proj.dtype \
+            or not out.is_contiguous():
+        raise KernelError("conv_heads: out must be contiguous [n, (heads + 2 kv heads) * head_cols] of the projection's type")
+    if rot:
+        for t in (cos, sin):
+            if t is None or t.dtype != torch.float32 or not t.is_contiguous() or t.shape[1] != rot // 2 or t.shape[0] < n:
+                raise KernelError("conv_heads: cos/sin must be contiguous float32 [n, rot / 2]")
+    page_size = 0
+    if slots is not None:
+        _i32(slots, "slots", n)
+        _, p_heads, page_size, p_hd = _check_pages(k_pages, v_pages, proj.dtype, "conv_heads")
+        if (p_heads, p_hd) != (n_kv_heads, head_cols):
+            raise KernelError("conv_heads: pages do not have this layer's kv heads and head size")
+    single = int(ctx.host["max_q_len"]) == 1
+    lib = _lib("shortconv")
+    _launch(lib, lib.gb_conv_heads, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(wconv), taps, _p(state),
+            _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots), _p(cos) if rot else None,
+            _p(sin) if rot else None, int(rot), float(eps), 1 if norm else 0, _p(out), out.stride(0), int(head_cols),
+            _p(slots), _p(k_pages) if slots is not None else None, _p(v_pages) if slots is not None else None, page_size, n,
+            n_heads, n_kv_heads, dim, vdim, 1 if single else 0, _stream())
+    if wconv is not None and taps > 1 and not single:
+        _launch(lib, lib.gb_conv_state, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(state), _p(ctx.q_start),
+                _p(ctx.q_len), _p(ctx.state_slots), ctx.num_seqs, channels, taps, _stream())
+
+
+# ------------------------------------------------------------------- routed experts
+MOE_MAX_EXPERTS = 512   # moe.hip: a lane of the routing wave holds eight experts
+MOE_MAX_TOP = 16
+
+
+def moe_route(z: torch.Tensor, n_experts: int, correction: Optional[torch.Tensor], top: int, scale: float, shared: bool,
+              combine: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """From router logits ``z`` (float32 [n, experts (+ 1)]): scores sigmoid(z); the ``top`` experts with the largest
+    score + correction (of equal ones the lower index); their weights score / (sum of the chosen scores + 1e-20) * scale.
+    ``ids`` int32 and ``weights`` float32 [n, top] receive the choice, ``combine`` float32 [n, experts (+ 1)] a row of
+    weights with zeros for the others; with ``shared``, its last column is sigmoid of z's last column."""
+    _dev(z, correction, combine, ids, weights)
+    n = z.shape[0]
+    cols = n_experts + (1 if shared else 0)
+    if z.dtype != torch.float32 or z.dim() != 2 or z.stride(1) != 1 or z.shape[1] < cols:
+        raise KernelError("moe_route: z must be float32 [n, experts (+ 1)] with dense rows")
+    _f32_rows(combine, (n, cols), "combine")
+    _f32_rows(weights, (n, top), "weights")
+    _i32(ids, "ids", n * top)
+    if correction is not None:
+        _f32_rows(correction, (n_experts,), "correction")
+    lib = _lib("moe")
+    _launch(lib, lib.gb_moe_route, _p(z), z.stride(0), n, n_experts, _p(correction), int(top), float(scale),
+            1 if shared else 0, _p(combine), _p(ids), _p(weights), _stream())
+
+
+def moe_gated_units(gate_up: torch.Tensor, combine: torch.Tensor, out: torch.Tensor, n_experts: int, ff: int) -> None:
+    """out[t, j] = silu(gate) * up * combine[t, expert of column j]: ``gate_up`` [n, 2 * I] holds all gate columns, then all
+    up columns; columns e * ff .. of a half are expert e's, those from experts * ff on the shared expert's (weight in the
+    last column of ``combine``)."""
+    _dev(gate_up, combine, out)
+    n, inter = out.shape
+    if gate_up.shape != (n, 2 * inter) or gate_up.stride(1) != 1 or not out.is_contiguous():
+        raise KernelError("moe_gated_units: gate_up must be [n, 2 I] and out contiguous [n, I]")
+    if combine.dtype != torch.float32 or not combine.is_contiguous() or combine.shape[0] != n:
+        raise KernelError("moe_gated_units: combine must be contiguous float32 [n, experts (+ 1)]")
+    lib = _lib("moe")
+    _launch(lib, lib.gb_moe_gated_units, _p(gate_up), dtype_code(gate_up), gate_up.stride(0), _p(combine), combine.shape[1],
+            _p(out), dtype_code(out), n, inter, n_experts, ff, _stream())
+
+
+# ------------------------------------------------------------------- small residual operations
+def embed_pairs(table: torch.Tensor, pairs: torch.Tensor, ctx, out: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int,
+                prev: torch.Tensor) -> None:
+    """out[i] = table[id_i] + pairs[(id_(i-1) * mul_prev + id_i * mul_cur) mod buckets], row ``buckets`` of ``pairs`` for
+    a request's first token; float32 [n, d] or [copies, n, d].  ``prev`` int32 [slots, 1]: the last token of each
+    request's earlier steps, read for the first row of a request that goes on and left for the next step."""
+    _dev(table, pairs, out, prev)
+    copies = out.shape[0] if out.dim() == 3 else 1
+    n, d = out.shape[-2:]
+    if out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous() or table.shape[1] != d \
+            or not pairs.is_contiguous() or tuple(pairs.shape) != (buckets + 1, d) or pairs.dtype != table.dtype:
+        raise KernelError("embed_pairs: out must be contiguous float32 [n, d], table [vocab, d], pairs [buckets + 1, d]")
+    if prev.dtype != torch.int32 or not prev.is_contiguous() or prev[0].numel() != 1:
+        raise KernelError("embed_pairs: prev must be contiguous int32, one entry a slot")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_embed_pairs, _p(table), _p(pairs), dtype_code(table), _p(ctx.token_ids), _p(out), n, d, table.shape[0],
+            int(buckets), int(mul_prev), int(mul_cur), _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0),
+            _p(ctx.state_slots), _p(prev), int(copies), _stream())
+
+
+def glu_clamped(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> None:
+    """out = g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); ``gate_up`` [n, 2 I]
+    (gate columns, then up columns) in float32 or the result's type."""
+    _dev(gate_up, out)
+    n, inter = out.shape
+    if gate_up.shape != (n, 2 * inter) or gate_up.stride(1) != 1 or not out.is_contiguous():
+        raise KernelError("glu_clamped: gate_up must be [n, 2 I] and out contiguous [n, I]")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_glu_clamped, _p(gate_up), dtype_code(gate_up), gate_up.stride(0), _p(out), dtype_code(out), n, inter,
+            float(limit), float(alpha), _stream())
+
+
+def axpy_rows(x: torch.Tensor, y: Optional[torch.Tensor] = None, alpha: float = 1.0, bias: Optional[torch.Tensor] = None) -> None:
+    """x[r, :] += alpha * y[r, :] + bias, all float32; ``y`` or ``bias`` may be None."""
+    _dev(x, y, bias)
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("axpy_rows: x must be contiguous float32 [n, d]")
+    if y is not None and (y.dtype != torch.float32 or not y.is_contiguous() or y.shape != x.shape):
+        raise KernelError("axpy_rows: y must be contiguous float32 of x's shape")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() != d):
+        raise KernelError("axpy_rows: bias must be contiguous float32 [d]")
+    lib = _lib("elementwise")
+    _launch(lib, lib.gb_axpy_rows, _p(x), _p(y), float(alpha), _p(bias), n, d, _stream())
 
 
 # ------------------------------------------------------------------------ products

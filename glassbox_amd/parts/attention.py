@@ -15,7 +15,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, TensorSpec, emit_target,
+from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, StateSpec, TensorSpec, emit_target,
                    needs_multiple_of_8, product, split_workspace)
 
 
@@ -233,3 +233,102 @@ class TiedValueAttention(Mixer):
         product(ctx, att, self.wo, residual, accumulate=not store)
         if self.bias_o is not None:
             ops.add_bias(residual, self.bias_o)
+
+
+def cache_head_cols(dim: int, vdim: int) -> int:
+    """Columns of a head in the pages of a layer whose keys have ``dim`` channels and whose values have ``vdim``: the
+    cache and the attention kernels work on heads of one size, so both are filled up with zeros (which change neither a
+    score nor a weighted sum) to the larger of the two, and on to a multiple of 16 where the matrix-core kernels then
+    take the head, else to a multiple of 8."""
+    most = max(dim, vdim)
+    cols = -(-most // 16) * 16
+    return cols if cols <= 128 else -(-most // 8) * 8
+
+
+class ShortConvAttention(Mixer):
+    """Grouped-query attention whose projections pass a short causal convolution over time before anything else:
+    q, k, v = W h; each channel of the three convolved over its request's tokens with ``taps`` weights (``q.conv`` ...,
+    [channels, taps], zeros before the first token; ``taps`` 0: no convolution); the first ``rot_dims`` channels of every
+    query and key head turned by the position in neighbouring pairs (2i, 2i + 1), frequencies base^(-2i / rot_dims);
+    with ``qk_norm`` every query and key head divided by its root mean square; scores q . k * scale over the last
+    ``window`` keys (0: all); softmax; output projection.  Key and value heads may differ in size (``dim``, ``vdim``).
+
+    The request's last taps - 1 projections are its state (``state_spec``), beside the pages of keys and values."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: Optional[float] = None,
+                 window: int = 0, taps: int = 0, rot_dims: int = 0, rot_base: float = 10000.0, qk_norm: bool = True,
+                 eps: float = 1e-5):
+        from .rotary import Rotary
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key heads")
+        if rot_dims % 2 or not 0 <= rot_dims <= dim:
+            raise ValueError(f"{rot_dims} rotated channels: an even number up to the key size {dim}")
+        self.width, self.n_heads, self.n_kv_heads, self.dim, self.vdim = width, n_heads, n_kv_heads, dim, vdim
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(dim)
+        self.window, self.taps, self.rot_dims = int(window), int(taps), int(rot_dims)
+        self.qk_norm, self.eps = bool(qk_norm), float(eps)
+        self.head_cols = cache_head_cols(dim, vdim)
+        self.channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
+        self.position = Rotary(rot_dims, rot_base) if rot_dims else None
+        self.cache_spec = CacheSpec(n_kv_heads, self.head_cols, WINDOW if window > 0 else FULL, self.window)
+        self.state_spec = StateSpec((self.taps - 1, self.channels), torch.float32, 0.0) if self.taps > 1 else None
+        self.wqkv = self.wo = self.wconv = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H, G, D, V = self.n_heads, self.n_kv_heads, self.dim, self.vdim
+        specs = {"q": TensorSpec((H * D, self.width)), "k": TensorSpec((G * D, self.width)),
+                 "v": TensorSpec((G * V, self.width)), "o": TensorSpec((self.width, H * V))}
+        if self.taps:
+            specs.update({"q.conv": TensorSpec((H * D, self.taps), kind="f32"), "k.conv": TensorSpec((G * D, self.taps), kind="f32"),
+                          "v.conv": TensorSpec((G * V, self.taps), kind="f32")})
+        return specs
+
+    def load(self, tensors):
+        parts = [tensors["q"], tensors["k"], tensors["v"]]
+        if self.channels % 8:   # rows of the product's result then begin at 16-byte words
+            parts.append(torch.zeros((8 - self.channels % 8, self.width), dtype=parts[0].dtype, device=parts[0].device))
+        self.wqkv = torch.cat(parts, 0)
+        # the output projection takes heads of head_cols columns, the columns beyond vdim being zero
+        o = tensors["o"]
+        wo = torch.zeros((self.width, self.n_heads, self.head_cols), dtype=o.dtype, device=o.device)
+        wo[:, :, :self.vdim] = o.view(self.width, self.n_heads, self.vdim)
+        self.wo = wo.view(self.width, self.n_heads * self.head_cols)
+        if self.taps:
+            self.wconv = torch.cat([tensors["q.conv"], tensors["k.conv"], tensors["v.conv"]], 0).float().contiguous()
+
+    def streamed_matrices(self):
+        return [self.wqkv, self.wo]
+
+    def problems(self, dtype, page_size):
+        out = []
+        if self.head_cols > ops.MAX_HEAD_DIM:
+            out.append(("dim", f"heads of {max(self.dim, self.vdim)} channels are above {ops.MAX_HEAD_DIM}, the largest head "
+                               f"the attention kernels take"))
+        if self.taps > ops.CONV_MAX_TAPS:
+            out.append(("taps", f"{self.taps} is above {ops.CONV_MAX_TAPS}, the longest convolution the kernel takes"))
+        return out
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        if cache is None or cache.k_pages is None or (self.taps > 1 and cache.state is None):
+            raise ValueError("ShortConvAttention needs a layer cache with pages (and state, with a convolution)")
+        n = h.shape[0]
+        H, G, hc = self.n_heads, self.n_kv_heads, self.head_cols
+        proj = ctx.buffer("conv_proj", (n, self.wqkv.shape[0]), ctx.dtype)
+        product(ctx, h, self.wqkv, proj)
+        cos, sin = self.position.table(ctx) if self.position is not None else (None, None)
+        heads = ctx.buffer("conv_heads", (n, (H + 2 * G) * hc), ctx.dtype)
+        slots = ctx.slots[cache.group] if cache.writable else None
+        direct = slots is not None and n <= ops.ROPE_PRODUCT_MAX_ROWS
+        ops.conv_heads(proj, self.wconv, cache.state, ctx, cos, sin, self.rot_dims, self.eps, self.qk_norm, heads, hc,
+                       slots if direct else None, cache.k_pages, cache.v_pages, H, G, self.dim, self.vdim)
+        if slots is not None and not direct:
+            # many rows: the kernel that takes a step's keys and values to their pages in whole lines
+            ops.rope_store(heads, None, None, slots, cache.k_pages, cache.v_pages, H, G, hc, rotate=False,
+                           portions=ctx.portions())
+        att = ctx.buffer("att", (n, H * hc), ctx.dtype)
+        paged_attention(ctx, heads[:, :H * hc], att, cache, H, self.scale, self.window)
+        product(ctx, att, self.wo, residual, accumulate=not store)

@@ -13,6 +13,9 @@ from __future__ import annotations
 
 from typing import Dict, Optional
 
+import torch
+
+from .. import ops
 from .base import Block, CacheSpec, FeedForward, LayerCache, Mixer, Norm, Normed, Part, StateSpec
 
 
@@ -85,4 +88,43 @@ class MixerOnlyBlock(Block):
 
     def forward(self, ctx, x, cache: Optional[LayerCache]):
         self.mixer.forward(ctx, self.mixer_norm.forward(ctx, x), x, cache)
+        return None
+
+
+class ParallelBlock(Block):
+    """One norm, and both sublayers read its rows: x += mult * (mixer(norm(x)) + feed-forward(norm(x))); the
+    feed-forward may be absent.  The sublayers' sum is made in a 32-bit buffer of its own (the mixer writes its rows
+    there, the feed-forward adds to them: ``accepts_store``) and goes into the residual in one pass."""
+    replayable = True
+    taped = True
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: Optional[FeedForward] = None, mult: float = 1.0,
+                 names=("norm1", "mix", "mlp")):
+        for part in (mixer,):
+            if not getattr(part, "accepts_store", False):
+                raise ValueError(f"{type(part).__name__} cannot write its rows instead of adding them (accepts_store)")
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+        self.mult = float(mult)
+        self.names = tuple(names)
+
+    def children(self) -> Dict[str, Part]:
+        out = {self.names[0]: self.norm, self.names[1]: self.mixer}
+        if self.ffn is not None:
+            out[self.names[2]] = self.ffn
+        return out
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return self.mixer.cache_spec
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return self.mixer.state_spec
+
+    def forward(self, ctx, x, cache: Optional[LayerCache]):
+        n, width = x.shape
+        h = self.norm.forward(ctx, x)
+        y = ctx.buffer("parallel_y", (n, width), torch.float32)
+        self.mixer.forward(ctx, h, y, cache, store=True)
+        if self.ffn is not None:
+            self.ffn.forward(ctx, h, y)
+        ops.axpy_rows(x, y, self.mult)
         return None

@@ -8,7 +8,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import Part, TensorSpec, needs_multiple_of_8, product
+from .base import LayerCache, Part, StateSpec, TensorSpec, needs_multiple_of_8, product
 
 
 class Embedding(Part):
@@ -27,6 +27,37 @@ class Embedding(Part):
     def forward(self, ctx, out):
         """``out`` [n, width], or [streams, n, width]: every stream starts as the embedding."""
         ops.embed(self.table, ctx.token_ids, out, self.scale)
+
+
+class PairHashEmbedding(Embedding):
+    """The token's row plus a row of a second table chosen by the token and the one before it:
+    row (previous token * mul_prev + token * mul_cur) mod buckets, and the table's last row (number ``buckets``) for a
+    request's first token.  The token before a step's first row is part of the request's state: one int32 a slot
+    (``state_spec``), which the model hands over as a cache layer of the embedding's own."""
+    replayable = True
+
+    def __init__(self, vocab: int, width: int, buckets: int, mul_prev: int, mul_cur: int,
+                 names=("weight", "pairs")):
+        super().__init__(vocab, width)
+        if buckets < 1:
+            raise ValueError(f"{buckets} buckets: at least one")
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.names = tuple(names)
+        self.pairs: Optional[torch.Tensor] = None
+        self.state_spec = StateSpec((1,), torch.int32, 0)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.names[0]: TensorSpec((self.vocab, self.width)),
+                self.names[1]: TensorSpec((self.buckets + 1, self.width))}
+
+    def load(self, tensors):
+        self.table = tensors[self.names[0]].contiguous()
+        self.pairs = tensors[self.names[1]].contiguous()
+
+    def forward(self, ctx, out, cache: Optional[LayerCache] = None):
+        if cache is None or cache.state is None:
+            raise ValueError("PairHashEmbedding needs its state (the token before each request's step)")
+        ops.embed_pairs(self.table, self.pairs, ctx, out, self.buckets, self.mul_prev, self.mul_cur, cache.state)
 
 
 class LMHead(Part):

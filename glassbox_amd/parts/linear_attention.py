@@ -186,3 +186,80 @@ class GatedLinearAttention(_LinearMixer):
         ops.gla_prep(proj, 0, self.qk_dim, low_off, self.w_a2, self.a2_bias, q32, k32, decay,
                      1.0 / math.sqrt(self.key_dim), self.tau, z=z)
         self._finish(ctx, proj, q32, k32, residual, cache, store, self.norm_weight, decay=decay)
+
+
+class MLSTM(Mixer):
+    """Matrix memory with exponential gates.  Per head, q = W_q h / sqrt(key size), k = W_k h, v = W_v h, a log input
+    gate i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = log sigmoid(cap tanh((W_f h + b_f) / cap)); with a
+    running maximum m (0 before the first token): m_t = max(f_t + m_(t-1), i_t),
+    S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T, n_t the same with k_t alone,
+    o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).  Each head's o is divided by its root mean square, the heads
+    side by side are multiplied by ``norm`` (a weight for every channel of every head) and by sigmoid(W_g h), and
+    projected by W_o.
+
+    It is the decayed-state recurrence of this module with a decay a token and head, keys scaled by the input gate's
+    factor, and n as one more value channel whose v is 1.  The state of a request and head is [value size + 2, key size]
+    float32: the columns of S, n, and a row whose first element is m.  Gates, m, the factors, q and k are 32-bit in both
+    precisions (the gates' projections are a product of their own with 32-bit results)."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, key_dim: int, value_dim: int, gate_cap: float, eps: float):
+        if not gate_cap > 0:
+            raise ValueError(f"the gates' cap must be positive, got {gate_cap}")
+        self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
+        self.gate_cap, self.eps = float(gate_cap), float(eps)
+        self.qk_dim, self.v_dim = n_heads * key_dim, n_heads * value_dim
+        self.state_spec = StateSpec((n_heads, value_dim + 2, key_dim), torch.float32, 0.0)
+        self.w_in = self.w_gates = self.wo = self.bias_i = self.bias_f = self.norm_weight = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H = self.n_heads
+        return {"q": TensorSpec((self.qk_dim, self.width)), "k": TensorSpec((self.qk_dim, self.width)),
+                "v": TensorSpec((self.v_dim, self.width)), "g": TensorSpec((self.v_dim, self.width)),
+                "o": TensorSpec((self.width, self.v_dim)), "norm": TensorSpec((self.v_dim,), kind="f32", init="ones"),
+                "i": TensorSpec((H, self.width)), "i.b": TensorSpec((H,), kind="f32", init="normal"),
+                "f": TensorSpec((H, self.width)), "f.b": TensorSpec((H,), kind="f32", init="normal")}
+
+    def load(self, tensors):
+        self.w_in = _LinearMixer._stack([tensors[n] for n in ("q", "k", "v", "g")])   # one product computes all four
+        self.w_gates = torch.cat([tensors["i"], tensors["f"]], 0).contiguous()
+        self.wo = tensors["o"].contiguous()
+        self.bias_i, self.bias_f = tensors["i.b"].contiguous(), tensors["f.b"].contiguous()
+        self.norm_weight = tensors["norm"].contiguous()
+
+    def streamed_matrices(self):
+        return [self.w_in, self.w_gates, self.wo]
+
+    def problems(self, dtype, page_size):
+        if self.key_dim > ops.LINEAR_MAX_KEY_DIM:
+            return [("dim", f"{self.key_dim} is above {ops.LINEAR_MAX_KEY_DIM}, the largest key size the recurrence kernel takes")]
+        return []
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        if cache is None or cache.state is None:
+            raise ValueError("MLSTM needs a layer cache with state")
+        n, H, dk, dv = h.shape[0], self.n_heads, self.key_dim, self.value_dim
+        proj = ctx.buffer("lin_proj", (n, self.w_in.shape[0]), ctx.dtype)
+        product(ctx, h, self.w_in, proj)
+        z = ctx.buffer("mlstm_z", (n, 2 * H), torch.float32)
+        product(ctx, h, self.w_gates, z)
+        coef = ctx.buffer("mlstm_coef", (n, H, 3), torch.float32)
+        ops.mlstm_gates(z, self.bias_i, self.bias_f, self.gate_cap, coef, cache.state, dv + 1, ctx, H)
+        q32 = ctx.buffer("lin_q", (n, self.qk_dim), torch.float32)
+        k32 = ctx.buffer("lin_k", (n, self.qk_dim), torch.float32)
+        decay = ctx.buffer("mlstm_decay", (n, H), torch.float32)
+        vext = ctx.buffer("mlstm_v", (n, H * (dv + 1)), ctx.dtype)
+        ops.mlstm_prep(proj, 0, self.qk_dim, 2 * self.qk_dim, coef, q32, k32, decay, vext, H, dk, dv, 1.0 / math.sqrt(dk))
+        o = ctx.buffer("mlstm_o", (n, H * (dv + 1)), torch.float32)
+        segments = ops.linear_scan_segments(int(ctx.host["max_q_len"]))
+        ws = None
+        if segments > 1:
+            ws = ctx.buffer("lin_segments", (ctx.num_seqs * segments * H * (dv + 2) * dk,), torch.float32)
+        ops.linear_scan(q32, k32, vext, o, cache.state, ctx, H, dk, dv + 1, token_decay=decay, segments=segments, workspace=ws)
+        gated = ctx.buffer("lin_gated", (n, self.v_dim), ctx.dtype)
+        g_off = 2 * self.qk_dim + self.v_dim
+        ops.mlstm_out(o, coef, proj[:, g_off:g_off + self.v_dim], self.norm_weight, gated, H, dv, self.eps)
+        product(ctx, gated, self.wo, residual, accumulate=not store)

@@ -74,3 +74,38 @@ class SwiGLU(FeedForward):
         ops.gemm(act, self.w_down, residual, accumulate=not store, emit=target,
                  workspace=split_workspace(ctx, n, self.width, self.intermediate))
         return handed_on
+
+
+class ClampedGLU(FeedForward):
+    """A gated unit whose halves are clamped: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
+    y = g * sigmoid(alpha * g) * (u + 1), output W_down y.  Gate and up rows are stacked so one product computes both;
+    its sums stay 32-bit until the unit has been applied."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, intermediate: int, limit: float, alpha: float = 1.702):
+        self.width, self.intermediate = width, intermediate
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"gate": TensorSpec((self.intermediate, self.width)), "up": TensorSpec((self.intermediate, self.width)),
+                "down": TensorSpec((self.width, self.intermediate))}
+
+    def load(self, tensors):
+        self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], 0)
+        self.w_down = tensors["down"].contiguous()
+
+    def streamed_matrices(self):
+        return [self.w_gate_up, self.w_down]
+
+    def forward(self, ctx, h, residual, store: bool = False):
+        n = h.shape[0]
+        gate_up = ctx.buffer("glu_gate_up", (n, 2 * self.intermediate), torch.float32)
+        product(ctx, h, self.w_gate_up, gate_up)
+        act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
+        ops.glu_clamped(gate_up, act, self.limit, self.alpha)
+        product(ctx, act, self.w_down, residual, accumulate=not store)
+        return None

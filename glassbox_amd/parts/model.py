@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import ops
-from .base import CacheSpec, LayerCache, Norm, Normed, Part, PreNormed, StateSpec
+from .base import CacheSpec, LayerCache, Norm, Normed, Part, PreNormed, StateSpec, TensorSpec
 from .embedding import Embedding, LMHead
 from .tape import LayerTapes
 
@@ -26,6 +26,29 @@ class LayerCall:
     block: int
     cache: Optional[int] = None   # cache layer this call writes and reads
     reads: Optional[int] = None   # or: cache layer of another call that this one only reads
+    enter: Optional[int] = None   # the number of the pass over a repeated run that begins with this call (``PassEntry``)
+
+
+class PassEntry(Part):
+    """What a model adds to the residual where a pass over a repeated run of layers begins: before every pass but
+    the first the embedding's output (the residual as it was before the first layer), and before every pass, the first
+    too, row t of ``step`` ([passes, width]), t the number of the pass.  32-bit."""
+    replayable = True
+
+    def __init__(self, passes: int, width: int, add_embedding: bool = True):
+        self.passes, self.width, self.add_embedding = int(passes), int(width), bool(add_embedding)
+        self.step: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"step": TensorSpec((self.passes, self.width), kind="f32", init="normal")}
+
+    def load(self, tensors):
+        self.step = tensors["step"].contiguous()
+
+    def forward(self, ctx, x, embedded, t: int) -> None:
+        if not 0 <= t < self.passes:
+            raise ValueError(f"pass {t} of {self.passes}")
+        ops.axpy_rows(x, embedded if (t > 0 and self.add_embedding) else None, 1.0, self.step[t])
 
 
 class DecoderModel(Part):
@@ -34,8 +57,12 @@ class DecoderModel(Part):
     def __init__(self, config, embedding: Embedding, blocks: Sequence[Part], schedule: Sequence[LayerCall],
                  final_norm: Norm, head: LMHead, names=("model.embed_tokens", "model.layers.{}", "model.norm", "lm_head"),
                  ignorable: Sequence[str] = (), arg_keys: Optional[Dict[str, str]] = None, sources=None,
-                 streams: Optional[int] = None):
+                 streams: Optional[int] = None, passes: Optional[PassEntry] = None, passes_name: str = "loop"):
         self.config = config
+        #: what is added to the residual where a pass over a repeated run begins (``LayerCall.enter``), or None
+        self.passes, self.passes_name = passes, passes_name
+        if passes is not None and streams is not None:
+            raise ValueError("a residual of several streams has no pass entries")
         #: None: one residual [n, width]; a number: the residual is so many streams, [streams, n, width], which the
         #: embedding fills alike and the blocks and the final norm take as such (parts.streams)
         self.streams = streams
@@ -62,6 +89,8 @@ class DecoderModel(Part):
             out[self.names[1].format(i)] = b
         out[self.names[2]] = self.final_norm
         out[self.names[3]] = self.head
+        if self.passes is not None:
+            out[self.passes_name] = self.passes
         return out
 
     def source_of(self, name: str):
@@ -87,20 +116,36 @@ class DecoderModel(Part):
         if sorted(owners) != list(range(self.num_cache_layers)):
             raise ValueError("cache layers must be numbered 0..n-1 without gaps")
         self._owners = owners
+        for pos, call in enumerate(self.schedule):
+            if call.enter is not None and self.passes is None:
+                raise ValueError(f"schedule entry {pos} begins a pass, and the model has no pass entry")
+        #: an embedding that keeps something of each request from step to step gets a cache layer of its own, the last
+        self.embedding_cache = self.num_cache_layers if getattr(self.embedding, "state_spec", None) is not None else None
 
     def cache_specs(self) -> List[Optional[CacheSpec]]:
         """What each cache layer holds: the block that writes it says."""
-        return [self.blocks[self.schedule[self._owners[c]].block].cache_spec() for c in range(self.num_cache_layers)]
+        out = [self.blocks[self.schedule[self._owners[c]].block].cache_spec() for c in range(self.num_cache_layers)]
+        return out + ([None] if self.embedding_cache is not None else [])
 
     def state_specs(self) -> List[Optional[StateSpec]]:
-        return [self.blocks[self.schedule[self._owners[c]].block].state_spec() for c in range(self.num_cache_layers)]
+        out = [self.blocks[self.schedule[self._owners[c]].block].state_spec() for c in range(self.num_cache_layers)]
+        return out + ([self.embedding.state_spec] if self.embedding_cache is not None else [])
 
     # the step ---------------------------------------------------------------------
     def forward(self, ctx, caches: Sequence[LayerCache]) -> torch.Tensor:
         """Runs the tokens of ``ctx`` through every scheduled layer; logits [wanted, vocab] float32."""
         shape = (ctx.n, self.width) if self.streams is None else (self.streams, ctx.n, self.width)
+        embedded = None
+        keep = self.passes is not None and self.passes.add_embedding
+        if keep:   # the embedding writes a second copy, which later passes add to the residual
+            shape = (2,) + shape
         x = ctx.buffer("x", shape, torch.float32)
-        self.embedding.forward(ctx, x)
+        if self.embedding_cache is not None:
+            self.embedding.forward(ctx, x, caches[self.embedding_cache])
+        else:
+            self.embedding.forward(ctx, x)
+        if keep:
+            x, embedded = x[0], x[1]
         pre = None   # what the block before prepared of this block's first norm
         if self._taped is None:
             self._taped = [b.all_taped() for b in self.blocks]
@@ -116,12 +161,18 @@ class DecoderModel(Part):
             else:
                 cache = None
             block = self.blocks[call.block]
+            if call.enter is not None:
+                self.passes.forward(ctx, x, embedded, call.enter)
+                pre = None   # (what the block before prepared was of the residual before this)
             handover = hasattr(block, "entry_norm")
             more = {}
             if handover:
-                after = self.blocks[self.schedule[i + 1].block] if i + 1 < len(self.schedule) else None
+                last = i + 1 == len(self.schedule)
+                after = None if last else self.blocks[self.schedule[i + 1].block]
+                if not last and self.schedule[i + 1].enter is not None:
+                    after = None   # the residual changes before the next block reads it: nothing to prepare
                 more = {"pre": pre, "emit": after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None}
-                if after is None and self._head_takes_prepared(ctx):
+                if last and self._head_takes_prepared(ctx):
                     # the last block prepares the final norm as it would the next block's first
                     more["emit"] = self.final_norm.emit_spec(ctx, ctx.n)
             if tapes is not None and self._taped[call.block]:

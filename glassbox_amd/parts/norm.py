@@ -1,5 +1,6 @@
 """RMS norm: out = g * (x / sqrt(mean(x^2) + eps)), sums in 32-bit
-(crates/glassbox-core/src/model.rs:94-100)."""
+(crates/glassbox-core/src/model.rs:94-100).  With ``offset`` the checkpoint stores the weight around zero and
+g = offset + w, added in 32-bit when the weights are loaded and kept in 32-bit."""
 from __future__ import annotations
 
 from typing import Dict, Optional, Tuple
@@ -14,16 +15,21 @@ class RMSNorm(Norm):
     replayable = True
     taped = True
 
-    def __init__(self, width: int, eps: float):
+    def __init__(self, width: int, eps: float, offset: float = 0.0):
         self.width = width
         self.eps = float(eps)
+        self.offset = float(offset)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
+        if self.offset:
+            # (offset + w rounded to bfloat16 would lose most of w: the sum stays 32-bit)
+            return {"weight": TensorSpec((self.width,), kind="f32", init="zeros")}
         return {"weight": TensorSpec((self.width,), kind="vector", init="ones")}
 
     def load(self, tensors):
-        self.weight = tensors["weight"].contiguous()
+        w = tensors["weight"]
+        self.weight = (w.float() + self.offset).contiguous() if self.offset else w.contiguous()
 
     def forward(self, ctx, x, rows=None, out_name="h"):
         m = x.shape[0] if rows is None else rows.numel()
