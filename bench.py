@@ -3,12 +3,18 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
-    python bench.py --design sagalorn [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
+    python bench.py --design sagalorn|dekinex [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
 
 ``--design sagalorn`` is another measurement with a line of its own: prefill and decode throughput of Sagalorn models
 whose layers have the sizes of the named shapes (a third of the layers each retention, windowed attention with kept
 first keys and gated linear attention, every one with a feed-forward, two residual streams), beside a Llama of the
 same width, heads, feed-forward, vocabulary and number of layers.
+
+``--design dekinex`` does the same for Dekinex models: attention behind a short convolution (four taps, half of each
+head rotated, a window of 1,024) and the matrix memory with exponential gates in turn, a dense gated unit with
+clamped halves in every other layer and routed experts in the rest (eight experts of a quarter of the dense size, two a
+token, and a shared one of half the dense size: as many multiply-adds a token as the dense layer), a pair table of
+65,536 rows.
 
 A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step``
 (which replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the
@@ -66,9 +72,30 @@ def sagalorn_like(shapes: dict, layers: int, window: int = 1024, keep_first: int
                 embedding={"scale": 1.0}, norm={"eps": shapes["rms_norm_eps"]}, layers=[kinds[i % 3] for i in range(layers)])
 
 
+def dekinex_like(shapes: dict, layers: int, window: int = 1024, experts: int = 8, top: int = 2) -> dict:
+    """A Dekinex configuration with the widths of a Llama one: the two mixers in turn; dense and routed feed-forwards in
+    turn, the routed ones with as many multiply-adds a token as the dense ones."""
+    d, H, G = shapes["hidden_size"], shapes["num_attention_heads"], shapes["num_key_value_heads"]
+    hd = shapes.get("head_dim") or d // H
+    ff = shapes["intermediate_size"]
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": experts, "top": top, "scale": 1.0}, "shared": {"ff": ff // 2}}
+    attention = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "conv": 4, "scale": hd ** -0.5,
+                 "rot": {"dims": hd // 2, "base": 10000.0}, "mask": {"size": window}}
+    memory = {"heads": H, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    kinds = [{"type": "attention", "mixer": attention, "mlp": dense}, {"type": "mlstm", "mixer": memory, "mlp": moe},
+             {"type": "attention", "mixer": attention, "mlp": moe}, {"type": "mlstm", "mixer": memory, "mlp": dense}]
+    return dict(architecture="Dekinex", vocab=shapes["vocab_size"], width=d, residual_mult=0.5, norm={"eps": shapes["rms_norm_eps"]},
+                embedding={"bigram": {"buckets": 65536, "mul_prev": 1000003, "mul_cur": 31}},
+                layers=[kinds[i % 4] for i in range(layers)])
+
+
+DESIGNS = {"sagalorn": ("Sagalorn", sagalorn_like), "dekinex": ("Dekinex", dekinex_like)}
+
+
 def design_bench(a) -> int:
     """Prefill (one step of 2,048 tokens) and decode (batch and context as given, tokens fed back from the device sampler)
-    of a Sagalorn model and of the Llama of the same sizes, one after the other on the same GPU; one JSON line."""
+    of a model of the design and of the Llama of the same sizes, one after the other on the same GPU; one JSON line."""
     import torch
     from glassbox_amd.build import source_version
     from glassbox_amd.config import config_from_dict
@@ -124,9 +151,12 @@ def design_bench(a) -> int:
     for size in a.design_sizes.split(","):
         shapes = SHAPES[DESIGN_SIZES[size]]
         llama = dict(shapes, num_hidden_layers=layers, max_position_embeddings=max(shapes["max_position_embeddings"], a.context + 1))
-        sizes[size] = {"sagalorn": measure(sagalorn_like(shapes, layers)), "llama": measure(llama),
+        sizes[size] = {a.design: measure(DESIGNS[a.design][1](shapes, layers)),
+                       "llama": {} if a.only_design else measure(llama),
                        "width": shapes["hidden_size"], "ff": shapes["intermediate_size"], "layers": layers}
-    print(json.dumps({"design": "Sagalorn", "beside": "LlamaForCausalLM", "dtype": a.dtype, "batch": a.batch, "context": a.context,
+        if a.only_design:
+            del sizes[size]["llama"]
+    print(json.dumps({"design": DESIGNS[a.design][0], "beside": "LlamaForCausalLM", "dtype": a.dtype, "batch": a.batch, "context": a.context,
                       "prefill_tokens": PREFILL_TOKENS, "steps": a.steps, "warmup": a.warmup, "sizes": sizes,
                       "meta": {"gpu": torch.cuda.get_device_name(0), "commit": source_version(),
                                "date": datetime.datetime.now(datetime.timezone.utc).strftime("%Y-%m-%dT%H:%M:%SZ")}}))
@@ -159,7 +189,8 @@ def main() -> int:
                     help="read a step's sampled tokens back before the next step is launched")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --only prefill, for profiling: a prompt of another length than the 2,048 tokens of the record")
-    ap.add_argument("--design", choices=["sagalorn"], default=None,
+    ap.add_argument("--only-design", action="store_true", help="with --design, for profiling: skip the Llama beside it")
+    ap.add_argument("--design", choices=sorted(DESIGNS), default=None,
                     help="instead of the record: models of this design at the sizes of --design-sizes beside Llamas of equal size")
     ap.add_argument("--design-sizes", default="360m,1.7b", help="out of " + ", ".join(DESIGN_SIZES))
     a = ap.parse_args()

@@ -963,3 +963,4 @@ GB_TAPED(gb_scale_rows)
 GB_TAPED(gb_gemm_plain)
 GB_TAPED(gb_glu_clamped)
 GB_TAPED(gb_axpy_rows)
+GB_TAPED(gb_embed_pairs)
