@@ -463,11 +463,21 @@ __global__ __launch_bounds__(256) void head_norm_gate_words_kernel(const float* 
 // b_t = exp(i_t - m_t), and n as one more value channel whose v is 1.  The gates are capped,
 // i = cap tanh(z_i / cap), f = log sigmoid(cap tanh(z_f / cap)), z the projections plus their biases.
 
+// The gates of every (token, head), side by side: coef[t, h] = (f, i, .) for the kernel below.
+__global__ void mlstm_gate_values_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ bias_i,
+                                         const float* __restrict__ bias_f, float cap, float* __restrict__ coef, int n, int nh) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n * nh) return;
+  const int t = idx / nh, h = idx % nh;
+  const float* row = z + (size_t)t * ldz;
+  coef[(size_t)idx * 3 + 1] = cap * tanhf((row[h] + (bias_i ? bias_i[h] : 0.f)) / cap);
+  coef[(size_t)idx * 3] = log_sigmoid(cap * tanhf((row[nh + h] + (bias_f ? bias_f[h] : 0.f)) / cap));
+}
+
 // One wave a (request, head): 64 tokens at a time, each lane its token's gates; m over the 64 by a scan of the pairs
 // (F, I) that stand for m -> max(F + m, I) (first (F1, I1), then (F2, I2): (F1 + F2, max(I1 + F2, I2))).  Writes
 // coef[t, h] = (a_t, b_t, exp(-m_t)) and leaves the request's last m in its state slot at `m_at` of the head's block.
-__global__ __launch_bounds__(kWave) void mlstm_gates_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ bias_i,
-                                                          const float* __restrict__ bias_f, float cap, float* __restrict__ coef,
+__global__ __launch_bounds__(kWave) void mlstm_gates_kernel(float* __restrict__ coef,
                                                           float* __restrict__ state, long long head_floats, long long m_at,
                                                           const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
                                                           const int32_t* __restrict__ pos0, const int32_t* __restrict__ state_slots,
@@ -476,15 +486,14 @@ __global__ __launch_bounds__(kWave) void mlstm_gates_kernel(const float* __restr
   const int start = q_start[seq], L = q_len[seq];
   float* mp = state + ((size_t)state_slots[seq] * nh + h) * head_floats + m_at;
   float carry = pos0[seq] == 0 ? 0.f : *mp;
-  const float bi = bias_i ? bias_i[h] : 0.f, bf = bias_f ? bias_f[h] : 0.f;
   for (int base = 0; base < L; base += kWave) {
     const int t = base + lane;
     const bool valid = t < L;
     float ig = -INFINITY, fg = 0.f;
     if (valid) {
-      const float* row = z + (size_t)(start + t) * ldz;
-      ig = cap * tanhf((row[h] + bi) / cap);
-      fg = log_sigmoid(cap * tanhf((row[nh + h] + bf) / cap));
+      const float* c = coef + ((size_t)(start + t) * nh + h) * 3;
+      fg = c[0];
+      ig = c[1];
     }
     float F = fg, I = ig;
 #pragma unroll
@@ -692,18 +701,21 @@ extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, in
 }
 
 // z [n, ldz] float32: the input gates' projections of the nh heads, then the forget gates'; biases float32 [nh] or nullptr;
-// coef [n, nh, 3] float32 receives (a_t, b_t, exp(-m_t)); the running maximum of head h of a request lives at
+// coef [n, nh, 3] float32 (n: the step's rows) receives (a_t, b_t, exp(-m_t)); the running maximum of head h of a request lives at
 // state[slot][h * head_floats + m_at].
 extern "C" int gb_mlstm_gates(const float* z, int ldz, const float* bias_i, const float* bias_f, float cap, float* coef,
                               float* state, long long head_floats, long long m_at, const int32_t* q_start,
                               const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
-                              hipStream_t stream) {
+                              int n, hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && ldz >= 2 * nh && cap > 0.f, "mlstm_gates: bad sizes requests=%d heads=%d ldz=%d cap=%g", n_seqs, nh, ldz, cap);
   GB_REQUIRE(head_floats > 0 && m_at >= 0 && m_at < head_floats, "mlstm_gates: the maximum lies outside its head's state");
   GB_REQUIRE(n_seqs <= 2147483647 && nh <= 65535, "mlstm_gates: too many heads for one launch");
-  if (n_seqs == 0) return 0;
-  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(n_seqs, nh), dim3(kWave), 0, stream, z, ldz, bias_i, bias_f, cap, coef, state,
-                     head_floats, m_at, q_start, q_len, pos0, state_slots, nh);
+  GB_REQUIRE(n >= 0 && (long long)n * nh < (1ll << 31), "mlstm_gates: too many (token, head) pairs");
+  if (n_seqs == 0 || n == 0) return 0;
+  hipLaunchKernelGGL(mlstm_gate_values_kernel, dim3((unsigned)((n * nh + 255) / 256)), dim3(256), 0, stream, z, ldz, bias_i, bias_f,
+                     cap, coef, n, nh);
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(n_seqs, nh), dim3(kWave), 0, stream, coef, state, head_floats, m_at, q_start, q_len,
+                     pos0, state_slots, nh);
   return launched("mlstm_gates");
 }
 

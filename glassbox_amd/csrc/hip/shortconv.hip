@@ -13,8 +13,9 @@
 //   pairs (2i, 2i + 1), i < rot / 2, of a query or key head:  (a, b) -> (a cos - b sin, b cos + a sin), angles from
 //   the step's table [n, rot / 2]; then the head divided by sqrt(mean of its dim squares + eps).
 //
-// One wave a (token, head); a lane takes pairs of neighbouring channels.  Everything is computed in 32-bit and
-// rounded once, when it is stored.
+// A few lanes a (token, head), as many as the head has pairs of neighbouring channels, so that a wave takes several
+// short heads; a lane takes a pair.  A token whose taps all lie among the step's rows reads no state.  Everything is
+// computed in 32-bit and rounded once, when it is stored.
 #include "common.h"
 
 using namespace gb;
@@ -24,74 +25,75 @@ GB_DEFINE_LAST_ERROR
 namespace {
 
 constexpr int kMaxTaps = 8;
-constexpr int kPairsLane = 2;   // heads of up to 256 channels
 
-template <typename T>
+// TAPS: the convolution's length (0: none).  LPU lanes a (token, head), a lane PPL pairs of neighbouring channels: heads
+// of up to 2 * LPU * PPL columns; a wave takes 64 / LPU heads.
+template <typename T, int TAPS, int LPU, int PPL>
 __global__ __launch_bounds__(4 * kWave) void conv_heads_kernel(
-    const T* __restrict__ proj, int stride, const float* __restrict__ wconv, int taps, float* __restrict__ state,
+    const T* __restrict__ proj, int stride, const float* __restrict__ wconv, float* __restrict__ state,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0,
     const int32_t* __restrict__ state_slots, const float* __restrict__ cosv, const float* __restrict__ sinv, int rot,
     float eps, int norm, T* __restrict__ out, int out_stride, int hd, const int32_t* __restrict__ slots,
     T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size, int nh, int nkv, int dim, int vdim, int channels,
     long long units, int update_state) {
-  const long long unit = (long long)blockIdx.x * 4 + threadIdx.x / kWave;
-  if (unit >= units) return;
+  constexpr int K = TAPS > 0 ? TAPS - 1 : 0;
+  constexpr int UPW = kWave / LPU;   // heads a wave
+  const int lane = threadIdx.x % kWave, li = lane % LPU;
+  const long long unit = ((long long)blockIdx.x * 4 + threadIdx.x / kWave) * UPW + lane / LPU;
+  const bool live = unit < units;
   const int heads = nh + 2 * nkv;
-  const int t = (int)(unit / heads), u = (int)(unit % heads), lane = threadIdx.x % kWave;
+  const int t = live ? (int)(unit / heads) : 0, u = live ? (int)(unit % heads) : 0;
   const bool is_q = u < nh, is_k = !is_q && u < nh + nkv;
   const int D = (is_q || is_k) ? dim : vdim;
   const int ch0 = is_q ? u * dim : is_k ? nh * dim + (u - nh) * dim : (nh + nkv) * dim + (u - nh - nkv) * vdim;
   const int seq = tok_seq[t], start = q_start[seq], first_pos = pos0[seq];
-  const int pos = first_pos + (t - start);
-  const int K = taps - 1;
-  float* st = (wconv && K > 0) ? state + (size_t)state_slots[seq] * K * channels : nullptr;
+  const int off = t - start;           // the token's place in its request's rows of this step
+  float* st = K > 0 ? state + (size_t)state_slots[seq] * K * channels : nullptr;
+  const T* row = proj + (size_t)t * stride;
 
-  float y[kPairsLane][2];
+  float y[PPL][2];
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < kPairsLane; ++j) {
+  for (int j = 0; j < PPL; ++j) {
+    const int p = li + j * LPU;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-      const int c = (lane + j * kWave) * 2 + e;
+      const int c = 2 * p + e;
       float acc = 0.f;
-      if (c < D) {
+      if (live && c < D) {
         const int ch = ch0 + c;
-        if (!wconv) {
-          acc = to_f(proj[(size_t)t * stride + ch]);
+        if (TAPS == 0) {
+          acc = to_f(row[ch]);
+        } else if (off >= K && !update_state) {   // every tap lies among the step's rows
+#pragma unroll
+          for (int jt = 0; jt < TAPS; ++jt)
+            acc = fmaf(wconv[(size_t)ch * TAPS + jt], to_f(proj[(size_t)(t - (K - jt)) * stride + ch]), acc);
         } else {
-          float old[kMaxTaps];   // the channel's slot, as far as this token needs it or has to move it
+          float old[K > 0 ? K : 1];   // the channel's slot: index i is the position `first_pos` - K + i
 #pragma unroll
-          for (int i = 0; i < kMaxTaps - 1; ++i) old[i] = 0.f;
-          if (st) {
+          for (int i = 0; i < K; ++i) old[i] = (update_state || i >= off) ? st[(size_t)i * channels + ch] : 0.f;
 #pragma unroll
-            for (int i = 0; i < kMaxTaps - 1; ++i)
-              if (i < K && (update_state || i >= t - start)) old[i] = st[(size_t)i * channels + ch];
-          }
-#pragma unroll
-          for (int jt = 0; jt < kMaxTaps; ++jt) {
-            if (jt >= taps) break;
+          for (int jt = 0; jt < TAPS; ++jt) {
             const int back = K - jt;   // how many tokens before this one
             float v = 0.f;
-            if (t - back >= start) v = to_f(proj[(size_t)(t - back) * stride + ch]);
-            else if (pos - back >= 0) {
-              const int idx = (t - start) + jt;   // = (pos - back) - first_pos + K
+            if (off >= back) {
+              v = to_f(proj[(size_t)(t - back) * stride + ch]);
+            } else if (first_pos + off - back >= 0) {
 #pragma unroll
-              for (int i = 0; i < kMaxTaps - 1; ++i)
-                if (i == idx) v = old[i];
+              for (int i = 0; i < K; ++i)
+                if (i == off + jt) v = old[i];   // = (position - back) - first_pos + K
             }
-            acc = fmaf(wconv[(size_t)ch * taps + jt], v, acc);
+            acc = fmaf(wconv[(size_t)ch * TAPS + jt], v, acc);
           }
-          if (update_state && st) {   // a step of single tokens: the slot moves on by one
+          if (update_state) {   // a step of single tokens: the slot moves on by one
 #pragma unroll
-            for (int i = 0; i < kMaxTaps - 1; ++i)
-              if (i < K) st[(size_t)i * channels + ch] = i + 1 < K ? old[i + 1] : to_f(proj[(size_t)t * stride + ch]);
+            for (int i = 0; i < K; ++i) st[(size_t)i * channels + ch] = i + 1 < K ? old[i + 1 < K ? i + 1 : 0] : to_f(row[ch]);
           }
         }
       }
       y[j][e] = acc;
     }
-    const int p = lane + j * kWave;
-    if (!(!is_q && !is_k) && 2 * p + 1 < rot && 2 * p + 1 < D) {
+    if (live && (is_q || is_k) && 2 * p + 1 < rot && 2 * p + 1 < D) {
       const float cs = cosv[(size_t)t * (rot / 2) + p], sn = sinv[(size_t)t * (rot / 2) + p];
       const float a = y[j][0], b = y[j][1];
       y[j][0] = a * cs - b * sn;
@@ -101,10 +103,12 @@ __global__ __launch_bounds__(4 * kWave) void conv_heads_kernel(
     ss = fmaf(y[j][1], y[j][1], ss);
   }
   float s = 1.f;
-  if (norm && (is_q || is_k)) {
-    ss = wave_sum(ss);
-    s = 1.0f / sqrtf(ss / (float)D + eps);
+  if (norm) {   // (value heads take part in the moves and keep s = 1)
+#pragma unroll
+    for (int o = LPU / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+    if (is_q || is_k) s = 1.0f / sqrtf(ss / (float)D + eps);
   }
+  if (!live) return;
   const int slot = (!is_q && slots) ? slots[t] : -1;
   const int piece = key_piece(hd);
   T* kb = nullptr;
@@ -117,13 +121,12 @@ __global__ __launch_bounds__(4 * kWave) void conv_heads_kernel(
   }
   T* orow = out + (size_t)t * out_stride + (size_t)u * hd;
 #pragma unroll
-  for (int j = 0; j < kPairsLane; ++j) {
+  for (int j = 0; j < PPL; ++j) {
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-      const int c = (lane + j * kWave) * 2 + e;
+      const int c = (li + j * LPU) * 2 + e;
       if (c >= hd) continue;
-      const float val = c < D ? y[j][e] * s : 0.f;
-      const T r = from_f<T>(val);
+      const T r = from_f<T>(c < D ? y[j][e] * s : 0.f);
       orow[c] = r;
       if (slot >= 0) {
         if (is_k) kb[key_offset(slot % page_size, c, page_size, piece)] = r;
@@ -171,7 +174,7 @@ extern "C" int gb_conv_heads(const void* proj, int dtype, int stride, const floa
                              int dim, int vdim, int update_state, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && dim > 0 && vdim > 0 && hd >= dim && hd >= vdim,
              "conv_heads: bad sizes n=%d heads=%d+%d dim=%d vdim=%d hd=%d", n, nh, nkv, dim, vdim, hd);
-  GB_REQUIRE(hd <= 2 * kWave * kPairsLane, "conv_heads: heads of %d columns are above %d", hd, 2 * kWave * kPairsLane);
+  GB_REQUIRE(hd <= 4 * kWave, "conv_heads: heads of %d columns are above %d", hd, 4 * kWave);
   const int channels = (nh + nkv) * dim + nkv * vdim;
   GB_REQUIRE(stride >= channels && out_stride >= (nh + 2 * nkv) * hd, "conv_heads: rows shorter than their heads");
   GB_REQUIRE(!wconv || (taps >= 1 && taps <= kMaxTaps && (taps == 1 || state)), "conv_heads: %d taps (at most %d), with the state", taps, kMaxTaps);
@@ -180,18 +183,49 @@ extern "C" int gb_conv_heads(const void* proj, int dtype, int stride, const floa
   GB_REQUIRE(tok_seq && q_start && pos0 && state_slots, "conv_heads: the step's tables are needed");
   if (n == 0) return 0;
   const long long units = (long long)n * (nh + 2 * nkv);
-  GB_REQUIRE((units + 3) / 4 < (1ll << 31), "conv_heads: too many heads for one launch");
-  const dim3 grid((unsigned)((units + 3) / 4));
-  if (dtype == kF32)
-    hipLaunchKernelGGL(conv_heads_kernel<float>, grid, dim3(4 * kWave), 0, stream, (const float*)proj, stride, wconv, taps, state,
-                       tok_seq, q_start, pos0, state_slots, cosv, sinv, rot, eps, norm, (float*)out, out_stride, hd, slots,
-                       (float*)k_pages, (float*)v_pages, page_size, nh, nkv, dim, vdim, channels, units, update_state);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(conv_heads_kernel<bf16>, grid, dim3(4 * kWave), 0, stream, (const bf16*)proj, stride, wconv, taps, state,
-                       tok_seq, q_start, pos0, state_slots, cosv, sinv, rot, eps, norm, (bf16*)out, out_stride, hd, slots,
-                       (bf16*)k_pages, (bf16*)v_pages, page_size, nh, nkv, dim, vdim, channels, units, update_state);
-  else
+  const int pairs = (hd + 1) / 2;
+  int lpu = 4;
+  while (lpu < pairs && lpu < kWave) lpu *= 2;
+  const int ppl = pairs > kWave ? 2 : 1;
+  const long long waves = (units + kWave / lpu - 1) / (kWave / lpu);
+  GB_REQUIRE((waves + 3) / 4 < (1ll << 31), "conv_heads: too many heads for one launch");
+  const dim3 grid((unsigned)((waves + 3) / 4));
+  const int tp = wconv ? taps : 0;
+#define GB_CONV(TT, TP, LPU, PPL)                                                                                            \
+  hipLaunchKernelGGL((conv_heads_kernel<TT, TP, LPU, PPL>), grid, dim3(4 * kWave), 0, stream, (const TT*)proj, stride, wconv,  \
+                     state, tok_seq, q_start, pos0, state_slots, cosv, sinv, rot, eps, norm, (TT*)out, out_stride, hd, slots,  \
+                     (TT*)k_pages, (TT*)v_pages, page_size, nh, nkv, dim, vdim, channels, units, update_state)
+#define GB_CONV_L(TT, TP)                                                  \
+  switch (ppl == 2 ? 128 : lpu) {                                          \
+    case 4: GB_CONV(TT, TP, 4, 1); break;                                  \
+    case 8: GB_CONV(TT, TP, 8, 1); break;                                  \
+    case 16: GB_CONV(TT, TP, 16, 1); break;                                \
+    case 32: GB_CONV(TT, TP, 32, 1); break;                                \
+    case 64: GB_CONV(TT, TP, 64, 1); break;                                \
+    default: GB_CONV(TT, TP, 64, 2); break;                                \
+  }
+#define GB_CONV_T(TT)                                                      \
+  switch (tp) {                                                            \
+    case 0: GB_CONV_L(TT, 0) break;                                        \
+    case 1: GB_CONV_L(TT, 1) break;                                        \
+    case 2: GB_CONV_L(TT, 2) break;                                        \
+    case 3: GB_CONV_L(TT, 3) break;                                        \
+    case 4: GB_CONV_L(TT, 4) break;                                        \
+    case 5: GB_CONV_L(TT, 5) break;                                        \
+    case 6: GB_CONV_L(TT, 6) break;                                        \
+    case 7: GB_CONV_L(TT, 7) break;                                        \
+    default: GB_CONV_L(TT, 8) break;                                       \
+  }
+  if (dtype == kF32) {
+    GB_CONV_T(float)
+  } else if (dtype == kBF16) {
+    GB_CONV_T(bf16)
+  } else {
     return fail("conv_heads: unknown dtype %d", dtype);
+  }
+#undef GB_CONV_T
+#undef GB_CONV_L
+#undef GB_CONV
   return launched("conv_heads");
 }
 

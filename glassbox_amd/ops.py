@@ -88,8 +88,8 @@ _SIGS = {
         "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                            C.c_longlong, _vp],
         # z, ldz, bias_i, bias_f, cap, coef, state, floats a head, where m lies, q_start, q_len, pos0, state slots,
-        # requests, heads, stream
-        "gb_mlstm_gates": [_vp, _i, _vp, _vp, _f, _vp, _vp, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _i, _i, _vp],
+        # requests, heads, rows, stream
+        "gb_mlstm_gates": [_vp, _i, _vp, _vp, _f, _vp, _vp, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
         # proj, dtype, stride, q_off, k_off, v_off, coef, q32, k32, decay, vext, n, heads, dk, dv, q_scale, stream
         "gb_mlstm_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
         # o, coef, gate, dtype, gate stride, w, out, n, heads, dv, eps, stream
@@ -759,7 +759,7 @@ def mlstm_gates(z: torch.Tensor, bias_i: Optional[torch.Tensor], bias_f: Optiona
     lib = _lib("linear_attention")
     _launch(lib, lib.gb_mlstm_gates, _p(z), z.stride(0), _p(bias_i), _p(bias_f), float(cap), _p(coef), _p(state),
             int(state.shape[2] * state.shape[3]), int(m_row * state.shape[3]), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0),
-            _p(ctx.state_slots), ctx.num_seqs, n_heads, _stream())
+            _p(ctx.state_slots), ctx.num_seqs, n_heads, n, _stream())
 
 
 def mlstm_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, coef: torch.Tensor, q32: torch.Tensor,
