@@ -106,10 +106,23 @@ constexpr int TBK = 64, TLD = TBK + 8;  // k-step; LDS row stride in elements (1
 constexpr int TCPR = TBK / 8;           // 16-byte chunks per row of a k-step
 constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 
-template <int WM, int WN, int DEPTH, int EPI, bool KFULL, typename CT>
+//
+// GROUPED: the rows of A fall into groups that each have a W of their own (the tokens of an expert).  Row tile
+// blockIdx.y is not rows [y BM, (y + 1) BM) but what grp.map says of it: three numbers a tile, the group (below zero: a
+// tile that this launch does not need), the tile's first row and the end of its group's rows, which takes the place of M.
+// The group's W begins grp.w_stride elements a group further on; with EPI_SILU_MUL its up rows lie grp.up_off rows
+// behind its gate rows.  grp.rows, if given, names the row of A behind each row of the product.
+struct Groups {
+  const int32_t* map;
+  const int32_t* rows;
+  long long w_stride;
+  int up_off;
+};
+
+template <int WM, int WN, int DEPTH, int EPI, bool KFULL, typename CT, bool GROUPED = false>
 __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
                                                          int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
-                                                         int k_slice) {
+                                                         int k_slice, Groups grp) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int CA = BM * TCPR / 256, CW = BN * TCPR / 256;  // chunks a thread moves per k-step
   if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
@@ -123,14 +136,24 @@ __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const 
   __shared__ __attribute__((aligned(16))) bf16 Ws[2][BN][TLD];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * BM;
+  int m0 = blockIdx.y * BM;
   const int half = N / 2;  // EPI_SILU_MUL: number of gate rows
+  int up_off = half;       // and how far behind its gate row an up row lies
+  if constexpr (GROUPED) {
+    const int32_t* tile = grp.map + 3 * blockIdx.y;
+    const int group = tile[0];
+    if (group < 0) return;
+    m0 = tile[1];
+    M = tile[2];
+    w += (size_t)group * grp.w_stride;
+    up_off = grp.up_off;
+  }
   // row of W behind row r of the workgroup's W tile (r = wn*32*WN + j*32 + column)
   auto w_row = [&](int r) -> int {
     if (EPI == EPI_SILU_MUL) {
       const int wv = r / 64, j = (r % 64) / 32, col = r % 32;
       const int n = blockIdx.x * 64 + wv * 32 + col;
-      return n < half ? (j ? half + n : n) : -1;
+      return n < half ? (j ? up_off + n : n) : -1;
     }
     const int n = blockIdx.x * BN + r;
     return n < N ? n : -1;
@@ -157,7 +180,11 @@ __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const 
   for (int ci = 0; ci < CT_; ++ci) {
     const int ch = tid + 256 * (ci < CA ? ci : ci - CA);
     if (ci < CA) {
-      src[ci] = a + (size_t)min(m0 + ch / TCPR, M - 1) * lda + (ch % TCPR) * 8;
+      int row = min(m0 + ch / TCPR, M - 1);
+      if constexpr (GROUPED) {
+        if (grp.rows) row = grp.rows[row];
+      }
+      src[ci] = a + (size_t)row * lda + (ch % TCPR) * 8;
     } else {
       src[ci] = w + (size_t)max(w_row(ch / TCPR), 0) * ldw + (ch % TCPR) * 8;
     }
@@ -333,10 +360,10 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   if (wn == (B) && depth == (D)) {                                                                                          \
     if (kfull)                                                                                                              \
       hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
-                         N, K, 0);                                                                                          \
+                         N, K, 0, Groups{});                                                                                          \
     else                                                                                                                    \
       hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,  \
-                         M, N, K, 0);                                                                                       \
+                         M, N, K, 0, Groups{});                                                                                       \
   }
   if (low) {
     depth = wn == 1 ? 2 : 1;
@@ -1043,7 +1070,7 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
 #define GB_S(WM, FULL)                                                                                                   \
   if (!ring && !streams && (plan.bm == 64 * WM) && kfull == FULL)                                                                   \
     hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI_STORE, FULL, float>), grid, block, 0, stream, a, lda, w, ldw, ws, \
-                       N, M, N, K, plan.k_slice);
+                       N, M, N, K, plan.k_slice, Groups{});
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
 #undef GB_S
   if (int rc = launched("gemm_bf16 (split k)")) return rc;
@@ -1790,6 +1817,40 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
 #undef GB_TL
 }
 
+// Products of groups of rows, each group with a W of its own (the tiled kernel's GROUPED form): `map` holds three
+// numbers for each of `tiles` row tiles of `tile_rows` (64 or 128) rows, as a kernel on the device laid them out; a
+// group's W starts w_stride elements behind the one before.  Epilogue 0 stores (bfloat16 or float32), 2 forms
+// silu(gate) * up from the N / 2 gate rows of a group and the up rows up_off rows behind them.
+extern "C" int gb_gemm_bf16_grouped(const void* a, int lda, const int32_t* rows, const void* w, int ldw, long long w_stride,
+                                    int up_off, void* c, int ldc, int c_dtype, const int32_t* map, int tiles, int tile_rows,
+                                    int N, int K, int epilogue, hipStream_t stream) {
+  GB_REQUIRE(tiles >= 0 && N > 0 && K > 0 && (tile_rows == 64 || tile_rows == 128), "gemm_bf16_grouped: bad sizes tiles=%d of %d rows, N=%d K=%d",
+             tiles, tile_rows, N, K);
+  GB_REQUIRE(K % 8 == 0 && ldw % 8 == 0 && lda % 8 == 0 && w_stride % 8 == 0 && lda >= K && ldw >= K,
+             "gemm_bf16_grouped: the inner size, the row strides and the distance between groups (%d, %d, %d, %lld) must keep rows 16-byte aligned",
+             K, lda, ldw, w_stride);
+  GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && map, "gemm_bf16_grouped: operands must be 16-byte aligned");
+  GB_REQUIRE(epilogue == EPI_STORE || (epilogue == EPI_SILU_MUL && N % 2 == 0 && c_dtype == kBF16),
+             "gemm_bf16_grouped: the epilogue is a store or silu(gate) * up into bfloat16, got %d", epilogue);
+  GB_REQUIRE(c_dtype == kF32 || c_dtype == kBF16, "gemm_bf16_grouped: unknown result dtype %d", c_dtype);
+  const int cols = epilogue == EPI_SILU_MUL ? N / 2 : N, bn = epilogue == EPI_SILU_MUL ? 64 : 128;
+  GB_REQUIRE(ldc >= cols && tiles <= 65535, "gemm_bf16_grouped: rows of C are shorter than the product's, or more than 65535 row tiles");
+  if (tiles == 0) return 0;
+  const Groups grp{map, rows, w_stride, up_off};
+  const dim3 grid((cols + bn - 1) / bn, tiles), block(256);
+  const bf16* A = (const bf16*)a;
+  const bf16* W = (const bf16*)w;
+  const bool kfull = K % TBK == 0;
+#define GB_G(WM, EPI, CT, FULL)                                                                                              \
+  if (tile_rows == 64 * WM && epilogue == EPI && kfull == FULL && (EPI == EPI_SILU_MUL || (c_dtype == kF32) == std::is_same_v<CT, float>)) \
+    hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI, FULL, CT, true>), grid, block, 0, stream, A, lda, W, ldw, (CT*)c, ldc, 0, N, K, 0, grp);
+#define GB_GG(WM, FULL) GB_G(WM, EPI_SILU_MUL, bf16, FULL) GB_G(WM, EPI_STORE, float, FULL) GB_G(WM, EPI_STORE, bf16, FULL)
+  GB_GG(1, true) GB_GG(1, false) GB_GG(2, true) GB_GG(2, false)
+#undef GB_GG
+#undef GB_G
+  return launched("gemm_bf16 (grouped)");
+}
+
 // The QKV product of a step of at most 64 rows with EPI_ROPE (see RopeExtras): c is the stacked rows
 // [M][(nh + 2 nkv) hd] (or [M][nh hd] with nkv == 0: queries only), bfloat16.  gamma / parts as in
 // gb_gemm_bf16 (the norm before the product).
@@ -1819,4 +1880,5 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
 
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_gemm_bf16)
+GB_TAPED(gb_gemm_bf16_grouped)
 GB_TAPED(gb_gemm_bf16_rope)

@@ -9,6 +9,14 @@
 // gate of an expert that every token uses).  `gated_units` turns the stacked gate and up projections of all experts
 // into act = silu(gate) * up * weight, so that one product with the experts' down matrices side by side gives the
 // weighted sum of the chosen experts' outputs (an expert not chosen contributes exact zeros).
+//
+// With many tokens a step, the experts run on the rows that chose them alone.  `sort` puts the (token, choice) entries
+// in the order of their experts (entries of an expert in the order of the tokens): rows[r] is the token behind sorted
+// row r, pos[t * top + k] the sorted row of token t's k-th choice, and `map` cuts the sorted rows into row tiles that
+// lie in one expert each (three numbers a tile: expert, first row, end of the expert's rows; the tiles past the last one
+// carry expert -1).  The products then go tile by tile with the tile's expert's matrices, and `combine` adds up, for
+// each token, its chosen experts' output rows times their weights in the order of the choices, and the shared
+// expert's row times its gate.
 #include "common.h"
 
 using namespace gb;
@@ -97,8 +105,8 @@ __global__ __launch_bounds__(4 * kWave) void route_kernel(const float* __restric
 }
 
 // act[t, j] = silu(g) * u * combine[t, expert of column j]: columns e * ff .. (e + 1) * ff - 1 are expert e's, the
-// columns from E * ff on the shared expert's (weight in column E of combine).  Rows of `gu`: all gate columns, then all
-// up columns.
+// columns from E * ff on the shared expert's (weight in column E of combine).  Rows of `gu`: the experts' gate columns,
+// the experts' up columns, then the shared expert's gate columns and its up columns.
 template <typename I, typename O>
 __global__ void gated_units_kernel(const I* __restrict__ gu, int ld, const float* __restrict__ combine, int cols, O* __restrict__ act,
                                    long long count, int inter, int E, int ff) {
@@ -106,15 +114,126 @@ __global__ void gated_units_kernel(const I* __restrict__ gu, int ld, const float
   if (idx >= count) return;
   const long long t = idx / inter;
   const int j = (int)(idx % inter);
-  const int e = j < E * ff ? j / ff : E;
+  const int routed = E * ff;
+  const int e = j < routed ? j / ff : E;
   const float w = combine[(size_t)t * cols + e];
   float y = 0.f;
   if (w != 0.f) {
     const I* row = gu + (size_t)t * ld;
-    const float g = to_f(row[j]), u = to_f(row[inter + j]);
+    const int at = j < routed ? j : 2 * routed + (j - routed), up = j < routed ? routed : inter - routed;
+    const float g = to_f(row[at]), u = to_f(row[at + up]);
     y = g / (1.0f + expf(-g)) * u * w;
   }
   act[idx] = from_f<O>(y);
+}
+
+// counts[e]: how many of the n * top entries chose expert e.  One workgroup an expert.
+__global__ __launch_bounds__(256) void count_kernel(const int32_t* __restrict__ ids, int entries, int32_t* __restrict__ counts) {
+  __shared__ int part[4];
+  const int e = blockIdx.x;
+  int mine = 0;
+  for (int i = threadIdx.x; i < entries; i += 256) mine += ids[i] == e;
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, kWave);
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
+}
+
+// Workgroup e places expert e's entries behind those of the experts before it, in the order of the entries, and writes
+// its row tiles; the last workgroup also marks the tiles that are left over.
+__global__ __launch_bounds__(256) void place_kernel(const int32_t* __restrict__ ids, int entries, int top, int E,
+                                                    const int32_t* __restrict__ counts, int tile_rows, int tiles,
+                                                    int32_t* __restrict__ rows, int32_t* __restrict__ pos,
+                                                    int32_t* __restrict__ map) {
+  __shared__ int part[4];
+  __shared__ int first_row, first_tile, all_tiles;
+  const int e = blockIdx.x, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (threadIdx.x == 0) {
+    int r = 0, t = 0, all = 0;
+    for (int o = 0; o < E; ++o) {
+      if (o == e) {
+        first_row = r;
+        first_tile = t;
+      }
+      r += counts[o];
+      t += (counts[o] + tile_rows - 1) / tile_rows;
+    }
+    all = t;
+    all_tiles = all;
+  }
+  __syncthreads();
+  const int base = first_row, mine = counts[e];
+  int placed = 0;
+  for (int i0 = 0; i0 < entries; i0 += 256) {
+    const int i = i0 + threadIdx.x;
+    const bool hit = i < entries && ids[i] == e;
+    const unsigned long long votes = __ballot(hit);
+    const int before = __popcll(votes & ((1ull << lane) - 1ull));
+    __syncthreads();   // the last round's sums have been read
+    if (lane == 0) part[wave] = __popcll(votes);
+    __syncthreads();
+    int ahead = 0;
+    for (int v = 0; v < wave; ++v) ahead += part[v];
+    if (hit) {
+      const int r = base + placed + ahead + before;
+      rows[r] = i / top;
+      pos[i] = r;
+    }
+    placed += part[0] + part[1] + part[2] + part[3];
+  }
+  const int my_tiles = (mine + tile_rows - 1) / tile_rows;
+  for (int j = threadIdx.x; j < my_tiles; j += 256) {
+    int32_t* t = map + 3 * (size_t)(first_tile + j);
+    t[0] = e;
+    t[1] = base + j * tile_rows;
+    t[2] = base + mine;
+  }
+  if (e == E - 1)
+    for (int j = all_tiles + threadIdx.x; j < tiles; j += 256) {
+      int32_t* t = map + 3 * (size_t)j;
+      t[0] = -1;
+      t[1] = 0;
+      t[2] = 0;
+    }
+}
+
+// out[t] (+)= sum over k of wts[t, k] * y[pos[t, k]]  +  gates[t * ldg] * y_shared[t]; four columns a thread.
+__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y, int ldy, const int32_t* __restrict__ pos,
+                                                      const float* __restrict__ wts, int top, const float* __restrict__ ysh,
+                                                      int ldsh, const float* __restrict__ gates, int ldg, float* __restrict__ out,
+                                                      int ldo, int accumulate, int n, int quads, int y_rows) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)n * quads) return;
+  const int t = (int)(idx / quads), c = (int)(idx % quads) * 4;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < top; ++k) {
+    const float w = wts[(size_t)t * top + k];
+    // an entry whose expert is none (a row of logits that are no numbers) was never placed: any row will do for it
+    const int r = min(max(pos[(size_t)t * top + k], 0), y_rows - 1);
+    const float4 v = *reinterpret_cast<const float4*>(y + (size_t)r * ldy + c);
+    acc.x += w * v.x;
+    acc.y += w * v.y;
+    acc.z += w * v.z;
+    acc.w += w * v.w;
+  }
+  if (ysh) {
+    const float g = gates[(size_t)t * ldg];
+    const float4 v = *reinterpret_cast<const float4*>(ysh + (size_t)t * ldsh + c);
+    acc.x += g * v.x;
+    acc.y += g * v.y;
+    acc.z += g * v.z;
+    acc.w += g * v.w;
+  }
+  float4* o = reinterpret_cast<float4*>(out + (size_t)t * ldo + c);
+  if (accumulate) {
+    const float4 old = *o;
+    acc.x += old.x;
+    acc.y += old.y;
+    acc.z += old.z;
+    acc.w += old.w;
+  }
+  *o = acc;
 }
 
 }  // namespace
@@ -149,5 +268,35 @@ extern "C" int gb_moe_gated_units(const void* gu, int in_dtype, int ld, const fl
   return launched("moe_gated_units");
 }
 
+// Row tiles that `sort` may need for n * top entries over E experts: every expert's last tile may be short.
+extern "C" int gb_moe_sort_tiles(int entries, int E, int tile_rows) { return entries / tile_rows + E; }
+
+extern "C" int gb_moe_sort(const int32_t* ids, int n, int top, int E, int tile_rows, int tiles, int32_t* counts, int32_t* rows,
+                           int32_t* pos, int32_t* map, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && top > 0 && E > 0 && tile_rows > 0 && (long long)n * top < (1ll << 31), "moe_sort: bad sizes n=%d top=%d experts=%d", n, top, E);
+  GB_REQUIRE(tiles >= gb_moe_sort_tiles(n * top, E, tile_rows), "moe_sort: %d row tiles, %d may be needed", tiles,
+             gb_moe_sort_tiles(n * top, E, tile_rows));
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(count_kernel, dim3(E), dim3(256), 0, stream, ids, n * top, counts);
+  hipLaunchKernelGGL(place_kernel, dim3(E), dim3(256), 0, stream, ids, n * top, top, E, counts, tile_rows, tiles, rows, pos, map);
+  return launched("moe_sort");
+}
+
+extern "C" int gb_moe_combine(const float* y, int ldy, const int32_t* pos, const float* wts, int top, const float* ysh, int ldsh,
+                              const float* gates, int ldg, float* out, int ldo, int accumulate, int n, int d, int y_rows, hipStream_t stream) {
+  GB_REQUIRE(y_rows >= (long long)n * top, "moe_combine: y holds %d rows for %d tokens of %d choices", y_rows, n, top);
+  GB_REQUIRE(n >= 0 && d > 0 && d % 4 == 0 && ldy % 4 == 0 && ldo % 4 == 0 && (!ysh || (ldsh % 4 == 0 && gates)) && ldy >= d && ldo >= d,
+             "moe_combine: rows of %d columns (strides %d, %d, %d) must be whole groups of four", d, ldy, ldsh, ldo);
+  GB_REQUIRE(((uintptr_t)y % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)ysh % 16 == 0), "moe_combine: rows must be 16-byte aligned");
+  if (n == 0) return 0;
+  const long long count = (long long)n * (d / 4);
+  GB_REQUIRE((count + 255) / 256 < (1ll << 31), "moe_combine: too many elements");
+  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, y, ldy, pos, wts, top, ysh, ldsh,
+                     gates, ldg, out, ldo, accumulate, n, d / 4, y_rows);
+  return launched("moe_combine");
+}
+
+GB_TAPED(gb_moe_sort)
+GB_TAPED(gb_moe_combine)
 GB_TAPED(gb_moe_route)
 GB_TAPED(gb_moe_gated_units)

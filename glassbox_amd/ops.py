@@ -76,6 +76,10 @@ _SIGS = {
         "gb_moe_route": [_vp, _i, _i, _i, _vp, _i, _f, _i, _vp, _vp, _vp, _vp],
         # gate_up, its dtype, ld, combine, its columns, act, its dtype, n, inter, experts, ff, stream
         "gb_moe_gated_units": [_vp, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+        # ids, n, top, experts, rows a tile, tiles, counts, rows, pos, map, stream
+        "gb_moe_sort": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp],
+        # y, ldy, pos, weights, top, y_shared, its stride, gates, their stride, out, ldo, accumulate, n, d, rows of y, stream
+        "gb_moe_combine": [_vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     },
     "streams": {
         # X, stream stride, streams, w_in, gamma, gamma dtype, rows, out, out dtype, sum, m, d, eps, mix, w_out, y, stream
@@ -110,6 +114,8 @@ _SIGS = {
         # emit_gamma, emit_gamma_dtype, emit_h, emit_ldh, emit_ss, parts, n_parts, split_ws, split_ws_floats, stream
         "gb_gemm_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp, _vp, _i, _vp,
                          C.c_longlong, _vp],
+        # a, lda, rows, w, ldw, distance between groups, up_off, c, ldc, c_dtype, map, tiles, rows a tile, N, K, epilogue, stream
+        "gb_gemm_bf16_grouped": [_vp, _i, _vp, _vp, _i, C.c_longlong, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _i, _vp],
         "gb_gemm_bf16_split_floats": [_i, _i, _i],
         "gb_gemm_bf16_emit_parts": [_i, _i],
         "gb_gemm_bf16_emit_mode": [_i, _i, _i],
@@ -884,9 +890,9 @@ def moe_route(z: torch.Tensor, n_experts: int, correction: Optional[torch.Tensor
 
 
 def moe_gated_units(gate_up: torch.Tensor, combine: torch.Tensor, out: torch.Tensor, n_experts: int, ff: int) -> None:
-    """out[t, j] = silu(gate) * up * combine[t, expert of column j]: ``gate_up`` [n, 2 * I] holds all gate columns, then all
-    up columns; columns e * ff .. of a half are expert e's, those from experts * ff on the shared expert's (weight in the
-    last column of ``combine``)."""
+    """out[t, j] = silu(gate) * up * combine[t, expert of column j]: ``gate_up`` [n, 2 * I] holds the experts' gate columns, the
+    experts' up columns, then the shared expert's gate columns and its up columns; columns e * ff .. of ``out`` are expert
+    e's, those from experts * ff on the shared expert's (weight in the last column of ``combine``)."""
     _dev(gate_up, combine, out)
     n, inter = out.shape
     if gate_up.shape != (n, 2 * inter) or gate_up.stride(1) != 1 or not out.is_contiguous():
@@ -899,6 +905,77 @@ def moe_gated_units(gate_up: torch.Tensor, combine: torch.Tensor, out: torch.Ten
 
 
 # ------------------------------------------------------------------- small residual operations
+def moe_sort_tiles(entries: int, n_experts: int, tile_rows: int) -> int:
+    """Row tiles that ``moe_sort`` may need: every expert's last tile may be short."""
+    return entries // tile_rows + n_experts
+
+
+def moe_sort(ids: torch.Tensor, n_experts: int, tile_rows: int, counts: torch.Tensor, rows: torch.Tensor, pos: torch.Tensor,
+             tile_map: torch.Tensor) -> None:
+    """Orders the entries of ``ids`` (int32 [n, top]) by expert, entries of an expert in the order of the tokens:
+    ``rows`` [n * top] receives the token behind each sorted row, ``pos`` [n, top] the sorted row of each entry, and
+    ``tile_map`` [tiles, 3] cuts the sorted rows into tiles of at most ``tile_rows`` rows of one expert (expert, first row,
+    end of the expert's rows; expert -1 for the tiles left over).  ``counts`` [experts] is scratch."""
+    _dev(ids, counts, rows, pos, tile_map)
+    n, top = ids.shape
+    _i32(ids, "ids", n * top)
+    _i32(counts, "counts", n_experts)
+    _i32(rows, "rows", n * top)
+    _i32(pos, "pos", n * top)
+    tiles = tile_map.shape[0]
+    _i32(tile_map, "tile_map", tiles * 3)
+    lib = _lib("moe")
+    _launch(lib, lib.gb_moe_sort, _p(ids), n, top, n_experts, tile_rows, tiles, _p(counts), _p(rows), _p(pos), _p(tile_map), _stream())
+
+
+def moe_combine(y: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor, y_shared: Optional[torch.Tensor],
+                gates: Optional[torch.Tensor], out: torch.Tensor, accumulate: bool) -> None:
+    """out[t] (+)= sum over k of weights[t, k] * y[pos[t, k]] + gates[t] * y_shared[t], all float32; ``gates`` may be a
+    column of a wider tensor."""
+    _dev(y, pos, weights, y_shared, gates, out)
+    n, top = weights.shape
+    d = out.shape[1]
+    for t, what in ((y, "y"), (out, "out"), (y_shared, "y_shared")):
+        if t is not None and (t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[1] != d):
+            raise KernelError(f"moe_combine: {what} must be float32 [rows, {d}] with dense rows")
+    if out.shape[0] != n or y.shape[0] < n * top or (y_shared is not None and (y_shared.shape[0] != n or gates is None or gates.shape[0] != n)):
+        raise KernelError("moe_combine: y holds a row for every entry, out, y_shared and gates a row for every token")
+    _f32_rows(weights, (n, top), "weights")
+    _i32(pos, "pos", n * top)
+    lib = _lib("moe")
+    _launch(lib, lib.gb_moe_combine, _p(y), y.stride(0), _p(pos), _p(weights), top, _p(y_shared),
+            y_shared.stride(0) if y_shared is not None else 0, _p(gates), gates.stride(0) if gates is not None else 0,
+            _p(out), out.stride(0), 1 if accumulate else 0, n, d, y.shape[0], _stream())
+
+
+def gemm_grouped_takes(a: torch.Tensor, w: torch.Tensor, group_stride: int) -> bool:
+    """Whether ``gemm_grouped`` serves these operands: bfloat16, 16-byte aligned rows and groups."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and group_stride % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_grouped(a: torch.Tensor, rows: Optional[torch.Tensor], w: torch.Tensor, group_stride: int, n_out: int,
+                 tile_map: torch.Tensor, tile_rows: int, out: torch.Tensor, silu_mul: bool = False, up_offset: int = 0) -> None:
+    """Products of groups of rows with a matrix of their own each.  Sorted row r of the product reads row ``rows[r]`` of
+    ``a`` (row r without ``rows``); ``tile_map`` (as ``moe_sort`` writes it) names each row tile's group and rows; group g
+    uses the ``n_out`` rows of ``w`` that begin ``g * group_stride`` elements into it.  ``silu_mul``: the group's rows
+    are n_out / 2 gate rows, with the up row of each ``up_offset`` rows behind it, and out = silu(gate) * up."""
+    _dev(a, rows, w, tile_map, out)
+    K = a.shape[1]
+    cols = n_out // 2 if silu_mul else n_out
+    if not gemm_grouped_takes(a, w, group_stride) or a.stride(1) != 1 or w.stride(1) != 1 or w.shape[1] < K:
+        raise KernelError("gemm_grouped: operands must be bfloat16 with dense, 16-byte aligned rows")
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[1] != cols or (silu_mul and out.dtype != torch.bfloat16):
+        raise KernelError(f"gemm_grouped: out must be [rows, {cols}] with dense rows (bfloat16 behind silu(gate) * up)")
+    tiles = tile_map.shape[0]
+    _i32(tile_map, "tile_map", tiles * 3)
+    if rows is not None:
+        _i32(rows, "rows")
+    lib = _lib("gemm_bf16")
+    _launch(lib, lib.gb_gemm_bf16_grouped, _p(a), a.stride(0), _p(rows), _p(w), w.stride(0), int(group_stride), int(up_offset),
+            _p(out), out.stride(0), dtype_code(out), _p(tile_map), tiles, tile_rows, n_out, K, 2 if silu_mul else 0, _stream())
+
+
 def embed_pairs(table: torch.Tensor, pairs: torch.Tensor, ctx, out: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int,
                 prev: torch.Tensor) -> None:
     """out[i] = table[id_i] + pairs[(id_(i-1) * mul_prev + id_i * mul_cur) mod buckets], row ``buckets`` of ``pairs`` for

@@ -5,10 +5,13 @@ chosen (the correction only chooses); their weights are s / (sum of the chosen s
 W_down (silu(W_gate h) * (W_up h)) without biases, and the output is the weighted sum of the chosen experts' outputs.
 A shared expert of the same form may run for every token, times sigmoid(W_sg h), one number a token.
 
-The experts' gate and up matrices are stacked by rows and their down matrices side by side, the shared expert's
-behind them.  One product gives every expert's gate and up sums; the unit's kernel multiplies each expert's columns by
-the token's weight for it, zero for an expert that was not chosen; one product with the down matrices then adds up
-exactly the chosen experts' outputs.
+The experts' gate matrices are stacked by rows, then their up matrices, then the shared expert's gate and up; the down
+matrices stand side by side, the shared expert's last.  A step of few tokens runs every expert on every token: one
+product gives every expert's gate and up sums; the unit's kernel multiplies each expert's columns by the token's weight
+for it, zero for an expert that was not chosen; one product with the down matrices then adds up exactly the chosen
+experts' outputs, and every matrix is read once.  A step of many tokens (``routed``) runs an expert on the tokens that
+chose it alone: the (token, choice) entries are put in the order of their experts on the device, the two products go
+over row tiles that lie in one expert each, and each token's chosen rows are added up with their weights.
 """
 from __future__ import annotations
 
@@ -17,7 +20,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, TensorSpec, product
+from .base import FeedForward, TensorSpec, product, split_workspace
 
 
 class RoutedExperts(FeedForward):
@@ -51,9 +54,11 @@ class RoutedExperts(FeedForward):
         return specs
 
     def load(self, tensors):
-        names = [f"e{e}" for e in range(self.n_experts)] + (["shared"] if self.shared_ff else [])
-        self.w_gate_up = torch.cat([tensors[f"{n}.gate"] for n in names] + [tensors[f"{n}.up"] for n in names], 0)
-        self.w_down = torch.cat([tensors[f"{n}.down"] for n in names], 1).contiguous()
+        names = [f"e{e}" for e in range(self.n_experts)]
+        shared = ["shared"] if self.shared_ff else []
+        self.w_gate_up = torch.cat([tensors[f"{n}.gate"] for n in names] + [tensors[f"{n}.up"] for n in names] +
+                                   [tensors[f"shared.{m}"] for m in ("gate", "up") if self.shared_ff], 0)
+        self.w_down = torch.cat([tensors[f"{n}.down"] for n in names + shared], 1).contiguous()
         router = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_ff else [])
         self.w_router = torch.cat(router, 0).contiguous()
         self.correction = tensors["correction"].contiguous() if self.has_correction else None
@@ -78,9 +83,46 @@ class RoutedExperts(FeedForward):
         ids = ctx.buffer("moe_ids", (n, self.top), torch.int32)
         weights = ctx.buffer("moe_weights", (n, self.top), torch.float32)
         ops.moe_route(z, E, self.correction, self.top, self.router_scale, bool(self.shared_ff), combine, ids, weights)
+        if self.routed(ctx, n):
+            return self._routed(ctx, h, residual, store, combine, ids, weights)
         gate_up = ctx.buffer("moe_gate_up", (n, 2 * self.inter), torch.float32)
         product(ctx, h, self.w_gate_up, gate_up)
         act = ctx.buffer("act", (n, self.inter), ctx.dtype)
         ops.moe_gated_units(gate_up, combine, act, E, self.expert_ff)
         product(ctx, act, self.w_down, residual, accumulate=not store)
+        return None
+
+    def routed(self, ctx, n: int) -> bool:
+        """Whether a step of n tokens runs the experts on their own tokens: where the sorted rows, every expert's last
+        tile of 64 filled up, are fewer than n rows for every expert, and the matrix-core products take the sizes."""
+        E, ff, d = self.n_experts, self.expert_ff, self.width
+        return (ctx.dtype == torch.bfloat16 and n > 64 and n * self.top + 64 * E < n * E
+                and d % 8 == 0 and ff % 8 == 0 and self.shared_ff % 8 == 0 and self.w_gate_up.data_ptr() % 16 == 0
+                and self.w_down.data_ptr() % 16 == 0)
+
+    def _routed(self, ctx, h, residual, store, combine, ids, weights):
+        n, E, ff, d, top = h.shape[0], self.n_experts, self.expert_ff, self.width, self.top
+        entries = n * top
+        tile_rows = 128 if entries >= 256 * E else 64
+        tiles = ops.moe_sort_tiles(entries, E, tile_rows)
+        counts = ctx.buffer("moe_counts", (E,), torch.int32)
+        rows = ctx.buffer("moe_rows", (entries,), torch.int32)
+        pos = ctx.buffer("moe_pos", (n, top), torch.int32)
+        tile_map = ctx.buffer("moe_tiles", (tiles, 3), torch.int32)
+        ops.moe_sort(ids, E, tile_rows, counts, rows, pos, tile_map)
+        act = ctx.buffer("act", (entries, ff), torch.bfloat16)
+        ops.gemm_grouped(h, rows, self.w_gate_up, ff * self.w_gate_up.stride(0), 2 * ff, tile_map, tile_rows, act,
+                         silu_mul=True, up_offset=E * ff)
+        y = ctx.buffer("moe_y", (entries, d), torch.float32)
+        ops.gemm_grouped(act, None, self.w_down, ff, d, tile_map, tile_rows, y)
+        y_shared = gates = None
+        if self.shared_ff:
+            act_shared = ctx.buffer("moe_act_shared", (n, self.shared_ff), torch.bfloat16)
+            w = self.w_gate_up[2 * E * ff:]
+            ops.gemm(h, w, act_shared, silu_mul=True, workspace=split_workspace(ctx, n, 2 * self.shared_ff, d))
+            y_shared = ctx.buffer("moe_y_shared", (n, d), torch.float32)
+            w = self.w_down[:, E * ff:]
+            ops.gemm(act_shared, w, y_shared, workspace=split_workspace(ctx, n, d, self.shared_ff))
+            gates = combine[:, E]
+        ops.moe_combine(y, pos, weights, y_shared, gates, residual, accumulate=not store)
         return None

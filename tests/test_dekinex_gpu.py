@@ -275,9 +275,76 @@ def test_the_router_and_the_gated_units():
                     row[E] = torch.sigmoid(z[t, E])
                 assert torch.allclose(combine[t].cpu().to(F64), row, atol=1e-6)
                 assert torch.allclose(wts[t].cpu().to(F64), weights, atol=1e-6)
-                g, u = gu[t, :inter], gu[t, inter:]
+                # the experts' gate columns, their up columns, then the shared expert's gate and up columns
+                g = torch.cat([gu[t, :E * ff], gu[t, 2 * E * ff:2 * E * ff + sff]])
+                u = torch.cat([gu[t, E * ff:2 * E * ff], gu[t, 2 * E * ff + sff:]])
                 per = torch.cat([row[:E].repeat_interleave(ff), row[E:].repeat_interleave(sff)]) if shared else row.repeat_interleave(ff)
                 assert torch.allclose(act[t].cpu().to(F64), g * torch.sigmoid(g) * u * per, atol=1e-5)
+
+
+def test_entries_sorted_by_expert_and_cut_into_tiles():
+    from glassbox_amd import ops
+    gen = torch.Generator().manual_seed(3)
+    for n, top, E, tile_rows in ((300, 2, 6, 64), (77, 1, 3, 64), (1000, 4, 9, 128), (130, 3, 70, 64), (64, 2, 2, 128)):
+        ids = torch.stack([torch.randperm(E, generator=gen)[:top] for _ in range(n)]).to(torch.int32)
+        if E > 4:
+            ids[ids == 1] = 0            # an expert that no token chooses
+        tiles = ops.moe_sort_tiles(n * top, E, tile_rows)
+        counts = torch.empty(E, dtype=torch.int32, device=DEV)
+        rows = torch.full((n * top,), -7, dtype=torch.int32, device=DEV)
+        pos = torch.full((n, top), -7, dtype=torch.int32, device=DEV)
+        tile_map = torch.full((tiles, 3), -7, dtype=torch.int32, device=DEV)
+        ops.moe_sort(ids.to(DEV), E, tile_rows, counts, rows, pos, tile_map)
+        flat = ids.flatten().tolist()
+        order = sorted(range(n * top), key=lambda i: (flat[i], i))      # by expert, entries of one in their own order
+        assert rows.tolist() == [i // top for i in order]
+        assert [pos.flatten().tolist()[i] for i in order] == list(range(n * top))
+        want, at = [], 0
+        for e in range(E):
+            c = flat.count(e)
+            want += [[e, at + j, at + c] for j in range(0, c, tile_rows)]
+            at += c
+        got = tile_map.tolist()
+        assert got[:len(want)] == want and all(t[0] == -1 for t in got[len(want):]) and len(want) <= tiles
+
+
+@pytest.mark.parametrize("n, d, E, top, ff, sff", [(300, 64, 6, 2, 16, 32), (129, 96, 3, 1, 24, 0), (700, 128, 16, 2, 64, 8),
+                                                  (1100, 72, 9, 4, 8, 24)])
+def test_experts_on_their_own_tokens_alone(n, d, E, top, ff, sff):
+    """A step of many tokens sorts them by expert; the same step through every expert (in two halves of few enough
+    tokens) and the plain implementation give the same rows.  One expert's down matrix is a hundred times the others',
+    so that a row that went to the wrong expert, or came back to the wrong token, shows."""
+    from glassbox_amd.engine.context import Workspace
+    from glassbox_amd.parts.moe import RoutedExperts
+    gen = torch.Generator().manual_seed(n + E)
+    part = RoutedExperts(d, E, top, ff, 1.7, sff)
+    w = {}
+    for name, spec in part.tensor_specs().items():
+        t = torch.randn(spec.shape, generator=gen) * (0.5 if name in ("router", "shared.sg") else d ** -0.5)
+        w[name] = t.to(torch.bfloat16) if len(spec.shape) == 2 else t * 0.1
+    w["e1.down"] = (w["e1.down"].float() * 100).to(torch.bfloat16)
+    part.load({k: v.to(DEV) for k, v in w.items()})
+    h = (torch.randn(n, d, generator=gen)).to(torch.bfloat16)
+    ctx = SimpleNamespace(dtype=torch.bfloat16, workspace=Workspace(DEV))
+    ctx.buffer = ctx.workspace.buffer
+    assert part.routed(ctx, n) and not part.routed(ctx, 40)
+    out = torch.full((n, d), 3.0, device=DEV)
+    part.forward(ctx, h.to(DEV), out, store=True)
+    again = torch.full((n, d), 1.0, device=DEV)
+    part.forward(ctx, h.to(DEV), again, store=False)
+    assert torch.equal(again - 1.0 - out, torch.zeros_like(out)) or float((again - 1.0 - out).abs().max()) < 1e-5 * float(out.abs().max())
+    small = torch.empty(n, d, device=DEV)
+    for a in range(0, n, 40):
+        part.forward(ctx, h[a:a + 40].to(DEV), small[a:a + 40], store=True)
+    wp = {"p." + k: v.to(F64) for k, v in w.items()}
+    mlp = {"router": {"experts": E, "top": top, "scale": 1.7}, "shared": {"ff": sff} if sff else None}
+    ref = pd.routed_experts(wp, "p.", mlp, h.to(F64), r=pd.bf16)
+    scale = float(ref.abs().max())
+    # a token whose choice hangs on the rounding of the router's sums may differ from the plain choice; both kernels'
+    # paths read the same choice
+    assert float((out.cpu().to(F64) - small.cpu().to(F64)).abs().max()) < 2e-2 * scale
+    close = ((out.cpu().to(F64) - ref).abs().amax(1) < 2e-2 * scale)
+    assert int(close.sum()) >= n - max(2, n // 100)
 
 
 def test_the_clamped_unit_and_the_scaled_add():
