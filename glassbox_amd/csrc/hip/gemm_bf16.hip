@@ -112,6 +112,20 @@ constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 // tile that this launch does not need), the tile's first row and the end of its group's rows, which takes the place of M.
 // The group's W begins grp.w_stride elements a group further on; with EPI_SILU_MUL its up rows lie grp.up_off rows
 // behind its gate rows.  grp.rows, if given, names the row of A behind each row of the product.
+// The gated unit of an EPI_SILU_MUL product, with the numbers that a clamped unit changes:
+// g' = min(g, limit), u' = clamp(u, -limit, limit), act = g' sigmoid(alpha g') (u' + plus).  As it stands here it is
+// silu(g) u to the bit.
+struct Glu {
+  float limit = INFINITY;
+  float alpha = 1.0f;
+  float plus = 0.0f;
+};
+__device__ __forceinline__ float gated_unit(float g, float u, const Glu& p) {
+  g = fminf(g, p.limit);
+  u = fminf(fmaxf(u, -p.limit), p.limit);
+  return g / (1.0f + __expf(-(p.alpha * g))) * (u + p.plus);
+}
+
 struct Groups {
   const int32_t* map;
   const int32_t* rows;
@@ -122,7 +136,7 @@ struct Groups {
 template <int WM, int WN, int DEPTH, int EPI, bool KFULL, typename CT, bool GROUPED = false>
 __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w,
                                                          int ldw, CT* __restrict__ c, int ldc, int M, int N, int K,
-                                                         int k_slice, Groups grp) {
+                                                         int k_slice, Groups grp, Glu glu) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int CA = BM * TCPR / 256, CW = BN * TCPR / 256;  // chunks a thread moves per k-step
   if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
@@ -295,7 +309,7 @@ __global__ __launch_bounds__(256, WN == 2 ? 2 : 1) void gemm_tiled_kernel(const 
       for (int r = 0; r < 16; ++r) {
         const int gm = m0 + wm * 32 * WM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
         const float g = acc[i][0][r], u = acc[i][WN - 1][r];
-        if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+        if (gm < M) c[(size_t)gm * ldc + gn] = (CT)gated_unit(g, u, glu);
       }
     return;
   }
@@ -341,7 +355,8 @@ inline void tiled_plan(int M, int N, int* wn, int* depth) {
 }
 
 template <int EPI, typename CT>
-int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream,
+                 Glu glu = Glu{}) {
   int wn, depth;
   tiled_plan(M, N, &wn, &depth);
   if (EPI == EPI_SILU_MUL) wn = 2;  // a wave's two column tiles are gate and up
@@ -360,10 +375,10 @@ int launch_tiled(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   if (wn == (B) && depth == (D)) {                                                                                          \
     if (kfull)                                                                                                              \
       hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, true, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, \
-                         N, K, 0, Groups{});                                                                                          \
+                         N, K, 0, Groups{}, glu);                                                                                          \
     else                                                                                                                    \
       hipLaunchKernelGGL((gemm_tiled_kernel<WM, (B), (D), EPI, false, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc,  \
-                         M, N, K, 0, Groups{});                                                                                       \
+                         M, N, K, 0, Groups{}, glu);                                                                                       \
   }
   if (low) {
     depth = wn == 1 ? 2 : 1;
@@ -423,7 +438,7 @@ template <int LEFT> __device__ __forceinline__ void vm_wait() {
 
 template <int EPI, typename CT>
 __global__ __launch_bounds__(RGM * RGN * 64, 1) void gemm_ring_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, int ldw,
-                                                           CT* __restrict__ c, int ldc, int M, int N, int K, int k_slice) {
+                                                           CT* __restrict__ c, int ldc, int M, int N, int K, int k_slice, Glu glu) {
   int bx = blockIdx.x, by = blockIdx.y;
   if (k_slice > 0) {  // split k: workgroup z of a tile sums its own slice of k into its own copy of C
     int z = blockIdx.z;
@@ -581,7 +596,7 @@ __global__ __launch_bounds__(RGM * RGN * 64, 1) void gemm_ring_kernel(const bf16
         for (int r = 0; r < 16; ++r) {
           const int gm = m0 + wm * RTM * 32 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
           const float g = acc[i][2 * p][r], u = acc[i][2 * p + 1][r];
-          if (gm < M) c[(size_t)gm * ldc + gn] = (CT)(g / (1.0f + __expf(-g)) * u);
+          if (gm < M) c[(size_t)gm * ldc + gn] = (CT)gated_unit(g, u, glu);
         }
     }
     return;
@@ -633,11 +648,12 @@ inline bool ring_pays(int epi, const void* a, int lda, const void* w, int ldw, i
 }
 
 template <int EPI, typename CT>
-int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream) {
+int launch_ring(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, hipStream_t stream,
+                Glu glu = Glu{}) {
   const int cols = EPI == EPI_SILU_MUL ? N / 2 : N, bn = EPI == EPI_SILU_MUL ? RBN / 2 : RBN;
   const dim3 grid((cols + bn - 1) / bn, (M + RBM - 1) / RBM), block(RGM * RGN * 64);
   GB_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, 0);
+  hipLaunchKernelGGL((gemm_ring_kernel<EPI, CT>), grid, block, 0, stream, a, lda, w, ldw, c, ldc, M, N, K, 0, glu);
   return launched("gemm_bf16 (ring)");
 }
 
@@ -1066,11 +1082,11 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   }
   if (ring)
     hipLaunchKernelGGL((gemm_ring_kernel<EPI_STORE, float>), dim3((N + RBN - 1) / RBN, (M + RBM - 1) / RBM, plan.slices), dim3(RGM * RGN * 64),
-                       0, stream, a, lda, w, ldw, ws, N, M, N, K, plan.k_slice);
+                       0, stream, a, lda, w, ldw, ws, N, M, N, K, plan.k_slice, Glu{});
 #define GB_S(WM, FULL)                                                                                                   \
   if (!ring && !streams && (plan.bm == 64 * WM) && kfull == FULL)                                                                   \
     hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI_STORE, FULL, float>), grid, block, 0, stream, a, lda, w, ldw, ws, \
-                       N, M, N, K, plan.k_slice, Groups{});
+                       N, M, N, K, plan.k_slice, Groups{}, Glu{});
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
 #undef GB_S
   if (int rc = launched("gemm_bf16 (split k)")) return rc;
@@ -1817,6 +1833,21 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
 #undef GB_TL
 }
 
+// A product of many rows (more than 64) whose epilogue is the clamped gated unit (see Glu): W stacks gate rows over
+// up rows as for epilogue 2, C is bfloat16 [M, N / 2].  The kernels that serve few rows have no such form; their callers
+// apply the unit in a pass of its own.
+extern "C" int gb_gemm_bf16_glu(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int M, int N, int K,
+                                float limit, float alpha, float plus, hipStream_t stream) {
+  GB_REQUIRE(M > 64 && N > 0 && N % 2 == 0 && K > 0 && K % 8 == 0, "gemm_bf16_glu: bad sizes M=%d N=%d K=%d (more than 64 rows)", M, N, K);
+  GB_REQUIRE(ldw % 8 == 0 && lda % 8 == 0 && lda >= K && ldw >= K && ldc >= N / 2, "gemm_bf16_glu: row strides (%d, %d, %d)", lda, ldw, ldc);
+  GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_glu: operands must be 16-byte aligned");
+  GB_REQUIRE(limit > 0.f, "gemm_bf16_glu: the limit must be positive");
+  const Glu glu{limit, alpha, plus};
+  if (ring_pays(EPI_SILU_MUL, a, lda, w, ldw, M, N, K))
+    return launch_ring<EPI_SILU_MUL, bf16>((const bf16*)a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, stream, glu);
+  return launch_tiled<EPI_SILU_MUL, bf16>((const bf16*)a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, stream, glu);
+}
+
 // Products of groups of rows, each group with a W of its own (the tiled kernel's GROUPED form): `map` holds three
 // numbers for each of `tiles` row tiles of `tile_rows` (64 or 128) rows, as a kernel on the device laid them out; a
 // group's W starts w_stride elements behind the one before.  Epilogue 0 stores (bfloat16 or float32), 2 forms
@@ -1843,7 +1874,7 @@ extern "C" int gb_gemm_bf16_grouped(const void* a, int lda, const int32_t* rows,
   const bool kfull = K % TBK == 0;
 #define GB_G(WM, EPI, CT, FULL)                                                                                              \
   if (tile_rows == 64 * WM && epilogue == EPI && kfull == FULL && (EPI == EPI_SILU_MUL || (c_dtype == kF32) == std::is_same_v<CT, float>)) \
-    hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI, FULL, CT, true>), grid, block, 0, stream, A, lda, W, ldw, (CT*)c, ldc, 0, N, K, 0, grp);
+    hipLaunchKernelGGL((gemm_tiled_kernel<WM, 2, 1, EPI, FULL, CT, true>), grid, block, 0, stream, A, lda, W, ldw, (CT*)c, ldc, 0, N, K, 0, grp, Glu{});
 #define GB_GG(WM, FULL) GB_G(WM, EPI_SILU_MUL, bf16, FULL) GB_G(WM, EPI_STORE, float, FULL) GB_G(WM, EPI_STORE, bf16, FULL)
   GB_GG(1, true) GB_GG(1, false) GB_GG(2, true) GB_GG(2, false)
 #undef GB_GG
@@ -1881,4 +1912,5 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_gemm_bf16)
 GB_TAPED(gb_gemm_bf16_grouped)
+GB_TAPED(gb_gemm_bf16_glu)
 GB_TAPED(gb_gemm_bf16_rope)

@@ -116,6 +116,8 @@ _SIGS = {
                          C.c_longlong, _vp],
         # a, lda, rows, w, ldw, distance between groups, up_off, c, ldc, c_dtype, map, tiles, rows a tile, N, K, epilogue, stream
         "gb_gemm_bf16_grouped": [_vp, _i, _vp, _vp, _i, C.c_longlong, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _i, _vp],
+        # a, lda, w, ldw, c, ldc, M, N, K, limit, alpha, plus, stream
+        "gb_gemm_bf16_glu": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _f, _f, _f, _vp],
         "gb_gemm_bf16_split_floats": [_i, _i, _i],
         "gb_gemm_bf16_emit_parts": [_i, _i],
         "gb_gemm_bf16_emit_mode": [_i, _i, _i],
@@ -1149,6 +1151,24 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
                                      workspace.numel() if workspace is not None else 0, _stream())
     else:
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
+
+
+GLU_PRODUCT_MIN_ROWS = 65
+
+
+def gemm_glu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, limit: float, alpha: float, plus: float = 1.0) -> None:
+    """out = g' * sigmoid(alpha g') * (u' + plus) with g' = min(a . gate, limit) and u' = clamp(a . up, -limit, limit),
+    formed where the product's tiles are finished: w stacks gate rows over up rows, all bfloat16, out [M, N / 2].  For
+    steps of at least ``GLU_PRODUCT_MIN_ROWS`` rows (the kernels of fewer rows have no such epilogue)."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or w.shape[1] != K
+            or out.shape != (M, N // 2) or N % 2 or M < GLU_PRODUCT_MIN_ROWS):
+        raise KernelError(f"gemm_glu: bfloat16 a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match, or rows are few")
+    lib = _lib("gemm_bf16")
+    _launch(lib, lib.gb_gemm_bf16_glu, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(out), _rows(out, "out"), M, N, K,
+            float(limit), float(alpha), float(plus), _stream())
 
 
 def gemm_takes(a: torch.Tensor, w: torch.Tensor) -> bool:

@@ -103,9 +103,13 @@ class ClampedGLU(FeedForward):
 
     def forward(self, ctx, h, residual, store: bool = False):
         n = h.shape[0]
-        gate_up = ctx.buffer("glu_gate_up", (n, 2 * self.intermediate), torch.float32)
-        product(ctx, h, self.w_gate_up, gate_up)
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
-        ops.glu_clamped(gate_up, act, self.limit, self.alpha)
+        if ctx.dtype == torch.bfloat16 and n >= ops.GLU_PRODUCT_MIN_ROWS and ops.gemm_takes(h, self.w_gate_up):
+            # the unit is applied where the product's tile is finished: gate_up never reaches memory
+            ops.gemm_glu(h, self.w_gate_up, act, self.limit, self.alpha)
+        else:
+            gate_up = ctx.buffer("glu_gate_up", (n, 2 * self.intermediate), torch.float32)
+            product(ctx, h, self.w_gate_up, gate_up)
+            ops.glu_clamped(gate_up, act, self.limit, self.alpha)
         product(ctx, act, self.w_down, residual, accumulate=not store)
         return None

@@ -347,6 +347,23 @@ def test_experts_on_their_own_tokens_alone(n, d, E, top, ff, sff):
     assert int(close.sum()) >= n - max(2, n // 100)
 
 
+@pytest.mark.parametrize("n, d, ff, limit", [(65, 64, 40, 0.7), (300, 96, 72, 2.0), (2048, 64, 3072, 1.0)])
+def test_the_clamped_unit_where_the_products_tiles_are_finished(n, d, ff, limit):
+    """Steps of many rows apply the unit in the product's kernel (the last case in the kernel of the largest tiles); the
+    gate's sums are spread so that many lie beyond the limit on either side."""
+    from glassbox_amd import ops
+    gen = torch.Generator().manual_seed(n)
+    h = torch.randn(n, d, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(2 * ff, d, generator=gen) * 2.0 * d ** -0.5).to(torch.bfloat16)
+    act = torch.empty(n, ff, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_glu(h.to(DEV), w.to(DEV), act, limit, 1.702)
+    gu = h.to(F64) @ w.to(F64).t()
+    g, u = gu[:, :ff].clamp(max=limit), gu[:, ff:].clamp(-limit, limit)
+    want = g * torch.sigmoid(1.702 * g) * (u + 1)
+    assert float((gu[:, :ff] > limit).double().mean()) > 0.05 and float((gu[:, ff:] < -limit).double().mean()) > 0.05
+    assert float((act.cpu().to(F64) - want).abs().max()) < 1e-2 * float(want.abs().max())
+
+
 def test_the_clamped_unit_and_the_scaled_add():
     from glassbox_amd import ops
     torch.manual_seed(8)
