@@ -136,6 +136,128 @@ __global__ __launch_bounds__(4 * kWave) void conv_heads_kernel(
   }
 }
 
+// The same for steps of many rows in bfloat16 whose heads are made of whole groups of eight channels (and that leave the
+// cache write to the page-store kernel): a lane takes eight neighbouring channels of a head, so that every access to the
+// rows is a 16-byte word, and `lpu` lanes (a power of two, at least hd / 8) a head; and it takes them for TT rows one
+// after the other, so that it reads its channels' taps once and each row of the projections once: the last taps - 1
+// rows wait in registers, whichever request they belong to, and a row whose request began fewer rows ago takes those
+// taps from the request's slot or as zeros instead.  The taps are added up in the order of the kernel above: the
+// convolution's sums are the same to the bit.
+template <int TAPS, int TT>
+__global__ __launch_bounds__(4 * kWave) void conv_heads_wide_kernel(
+    const bf16* __restrict__ proj, int stride, const float* __restrict__ wconv, const float* __restrict__ state,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slots, const float* __restrict__ cosv, const float* __restrict__ sinv, int rot,
+    float eps, int norm, bf16* __restrict__ out, int out_stride, int hd, int nh, int nkv, int dim, int vdim, int channels,
+    long long units, int lpu, int n) {
+  constexpr int K = TAPS > 0 ? TAPS - 1 : 0;
+  constexpr int NW = TAPS > 0 ? TAPS : 1;
+  const int lane = threadIdx.x % kWave, li = lane % lpu;
+  const long long unit = ((long long)blockIdx.x * 4 + threadIdx.x / kWave) * (kWave / lpu) + lane / lpu;
+  const int c0 = li * 8;   // the first of the lane's eight columns of its head
+  const bool live = unit < units && c0 < hd;
+  const int heads = nh + 2 * nkv;
+  const int t0 = live ? (int)(unit / heads) * TT : 0, u = live ? (int)(unit % heads) : 0;
+  const bool is_q = u < nh, is_k = !is_q && u < nh + nkv;
+  const int D = (is_q || is_k) ? dim : vdim;
+  const int ch = (is_q ? u * dim : is_k ? nh * dim + (u - nh) * dim : (nh + nkv) * dim + (u - nh - nkv) * vdim) + c0;
+  const bool has = live && c0 < D;
+
+  float w[8 * NW];      // [channel][tap], as they lie in memory
+  float win[NW][8];     // win[j]: the projections of row t - K + j
+#pragma unroll
+  for (int i = 0; i < 8 * NW; ++i) w[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) win[j][c] = 0.f;
+  if (has) {
+    if (TAPS > 0) {
+#pragma unroll
+      for (int i = 0; i < 2 * TAPS; ++i) {
+        const float4 q = *reinterpret_cast<const float4*>(wconv + (size_t)ch * TAPS + 4 * i);
+        w[4 * i] = q.x, w[4 * i + 1] = q.y, w[4 * i + 2] = q.z, w[4 * i + 3] = q.w;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) {   // rows t0 - K .. t0 - 1 of the step, as far as it has them
+      const int r = t0 - K + j;
+      if (r >= 0) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(proj + (size_t)r * stride + ch);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) win[j + 1][c] = (float)x[c];
+      }
+    }
+  }
+#pragma unroll 1
+  for (int it = 0; it < TT; ++it) {
+    const int t = t0 + it;
+    const bool row = live && t < n;
+    float y[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) y[c] = 0.f;
+    if (row && has) {
+#pragma unroll
+      for (int j = 0; j < K; ++j)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) win[j][c] = win[j + 1][c];
+      const bf16x8 x = *reinterpret_cast<const bf16x8*>(proj + (size_t)t * stride + ch);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) win[K][c] = (float)x[c];
+      if (TAPS == 0) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) y[c] = win[0][c];
+      } else {
+        const int seq = tok_seq[t], off = t - q_start[seq], first_pos = pos0[seq];
+#pragma unroll
+        for (int jt = 0; jt < TAPS; ++jt) {
+          const int back = K - jt;   // how many tokens before this one
+          float v[8];
+#pragma unroll
+          for (int c = 0; c < 8; ++c) v[c] = win[jt][c];
+          if (off < back) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) v[c] = 0.f;
+            if (first_pos + off - back >= 0) {   // in the request's slot, at index off + jt
+              const float* st = state + ((size_t)state_slots[seq] * K + (off + jt)) * channels + ch;
+              const float4 lo = *reinterpret_cast<const float4*>(st), hi = *reinterpret_cast<const float4*>(st + 4);
+              v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+            }
+          }
+#pragma unroll
+          for (int c = 0; c < 8; ++c) y[c] = fmaf(w[c * NW + jt], v[c], y[c]);
+        }
+      }
+      if (is_q || is_k) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int p = c0 / 2 + i;
+          if (2 * p + 1 < rot) {
+            const float cs = cosv[(size_t)t * (rot / 2) + p], sn = sinv[(size_t)t * (rot / 2) + p];
+            const float a = y[2 * i], b = y[2 * i + 1];
+            y[2 * i] = a * cs - b * sn;
+            y[2 * i + 1] = b * cs + a * sn;
+          }
+        }
+      }
+    }
+    float s = 1.f;
+    if (norm) {   // (value heads take part in the moves and keep s = 1)
+      float ss = 0.f;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) ss = fmaf(y[c], y[c], ss);
+      for (int o = lpu / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+      if (is_q || is_k) s = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    if (row) {
+      bf16x8 r;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) r[c] = (bf16)(y[c] * s);   // (columns from D on are zero already)
+      *reinterpret_cast<bf16x8*>(out + (size_t)t * out_stride + (size_t)u * hd + c0) = r;
+    }
+  }
+}
+
 // The state after a step with prompt portions: a thread a (request, channel) reads what it keeps of the old slot and
 // of the step's rows, then writes.
 template <typename T>
@@ -183,6 +305,35 @@ extern "C" int gb_conv_heads(const void* proj, int dtype, int stride, const floa
   GB_REQUIRE(tok_seq && q_start && pos0 && state_slots, "conv_heads: the step's tables are needed");
   if (n == 0) return 0;
   const long long units = (long long)n * (nh + 2 * nkv);
+  const int tp = wconv ? taps : 0;
+  if (dtype == kBF16 && !slots && !update_state && n > 64 && dim % 8 == 0 && vdim % 8 == 0 && hd % 8 == 0 && hd <= 8 * kWave &&
+      stride % 8 == 0 && out_stride % 8 == 0 && (uintptr_t)proj % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+      (uintptr_t)wconv % 16 == 0 && (uintptr_t)state % 16 == 0) {
+    int lpu = 1;
+    while (lpu * 8 < hd) lpu *= 2;
+    // eight rows a lane where that still leaves the chip a few thousand waves, else two
+    const long long units8 = (long long)((n + 7) / 8) * (nh + 2 * nkv);
+    const int tt = (units8 + kWave / lpu - 1) / (kWave / lpu) >= 2048 ? 8 : 2;
+    const long long wide_units = (long long)((n + tt - 1) / tt) * (nh + 2 * nkv);
+    const long long waves = (wide_units + kWave / lpu - 1) / (kWave / lpu);
+    GB_REQUIRE((waves + 3) / 4 < (1ll << 31), "conv_heads: too many heads for one launch");
+    const dim3 grid((unsigned)((waves + 3) / 4));
+#define GB_WIDE_T(TP, TT)                                                                                                    \
+  hipLaunchKernelGGL((conv_heads_wide_kernel<TP, TT>), grid, dim3(4 * kWave), 0, stream, (const bf16*)proj, stride, wconv,     \
+                     state, tok_seq, q_start, pos0, state_slots, cosv, sinv, rot, eps, norm, (bf16*)out, out_stride, hd, nh,   \
+                     nkv, dim, vdim, channels, wide_units, lpu, n)
+#define GB_WIDE(TP)                     \
+  case TP:                              \
+    if (tt == 8) GB_WIDE_T(TP, 8);      \
+    else GB_WIDE_T(TP, 2);              \
+    break;
+    switch (tp) {
+      GB_WIDE(0) GB_WIDE(1) GB_WIDE(2) GB_WIDE(3) GB_WIDE(4) GB_WIDE(5) GB_WIDE(6) GB_WIDE(7) GB_WIDE(8)
+    }
+#undef GB_WIDE
+#undef GB_WIDE_T
+    return launched("conv_heads (wide)");
+  }
   const int pairs = (hd + 1) / 2;
   int lpu = 4;
   while (lpu < pairs && lpu < kWave) lpu *= 2;
@@ -190,7 +341,6 @@ extern "C" int gb_conv_heads(const void* proj, int dtype, int stride, const floa
   const long long waves = (units + kWave / lpu - 1) / (kWave / lpu);
   GB_REQUIRE((waves + 3) / 4 < (1ll << 31), "conv_heads: too many heads for one launch");
   const dim3 grid((unsigned)((waves + 3) / 4));
-  const int tp = wconv ? taps : 0;
 #define GB_CONV(TT, TP, LPU, PPL)                                                                                            \
   hipLaunchKernelGGL((conv_heads_kernel<TT, TP, LPU, PPL>), grid, dim3(4 * kWave), 0, stream, (const TT*)proj, stride, wconv,  \
                      state, tok_seq, q_start, pos0, state_slots, cosv, sinv, rot, eps, norm, (TT*)out, out_stride, hd, slots,  \

@@ -139,6 +139,59 @@ def test_convolved_rotated_normed_heads_in_portions(H, G, dk, dv, taps, rot, dty
                     assert torch.equal(kept[i], data[r][p])
 
 
+@pytest.mark.parametrize("H, G, dk, dv, taps, rot, times", [
+    (4, 2, 64, 64, 4, 32, 1), (2, 1, 128, 80, 3, 128, 1), (3, 3, 16, 24, 8, 6, 1), (2, 2, 72, 40, 1, 0, 1), (5, 1, 32, 48, 0, 10, 1),
+    (1, 1, 24, 8, 2, 24, 1), (32, 32, 64, 64, 4, 8, 14)])   # (the last: enough rows and heads for eight rows a lane)
+def test_steps_of_many_rows_take_eight_channels_a_lane(H, G, dk, dv, taps, rot, times):
+    """Steps of more than 64 rows in bfloat16 whose heads are whole groups of eight channels, without the cache write:
+    two steps, requests that begin, one that goes on from its slot (its first rows read the slot), into slots that held
+    garbage; against the plain functions, and the slots after each step."""
+    from glassbox_amd import ops
+    from glassbox_amd.parts.attention import cache_head_cols
+    torch.manual_seed(dk + dv + taps)
+    base, eps, dtype = 100.0, 1e-5, torch.bfloat16
+    C, hc = (H + G) * dk + G * dv, cache_head_cols(dk, dv)
+    m = times
+    lens = {0: 110 * m + 3, 1: 30 * m, 2: 50 * m}
+    steps = [[(0, 0, 70 * m + 1), (1, 0, 30 * m)], [(0, 70 * m + 1, 110 * m + 3), (2, 0, 50 * m)]]
+    slots = {0: 2, 1: 0, 2: 3}
+    wconv = torch.randn(C, taps) if taps else None
+    state = torch.full((5, max(taps - 1, 1), C), 55.0, device=DEV) if taps > 1 else None
+    data, want = {}, {}
+    for r, T in lens.items():
+        u = torch.randn(T, C).to(dtype).to(F64)
+        data[r] = u
+        y = pd.short_convolution(u, wconv.to(F64)) if taps else u
+        q, k, v = y[:, :H * dk].view(T, H, dk), y[:, H * dk:(H + G) * dk].view(T, G, dk), y[:, (H + G) * dk:].view(T, G, dv)
+        want[r] = (pd.unit_rms(pd.rotate_neighbours(q, rot, base), eps), pd.unit_rms(pd.rotate_neighbours(k, rot, base), eps), v)
+    for rows in steps:
+        ctx = _step_ctx(rows, slots)
+        n = sum(b - a for _, a, b in rows)
+        assert n > 64
+        positions = [p for _, a, b in rows for p in range(a, b)]
+        ang = torch.tensor(positions, dtype=F64)[:, None] * torch.tensor([base ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=F64) \
+            if rot else None
+        proj = torch.zeros(n, C + 8, dtype=dtype, device=DEV)   # rows wider than their heads
+        proj[:, :C] = _dev(torch.cat([data[r][a:b] for r, a, b in rows], 0), dtype)
+        out = torch.full((n, (H + 2 * G) * hc), 9.0, dtype=dtype, device=DEV)
+        ops.conv_heads(proj, _dev(wconv) if taps else None, state, ctx, _dev(ang.cos()) if rot else None,
+                       _dev(ang.sin()) if rot else None, rot, eps, True, out, hc, None, None, None, H, G, dk, dv)
+        got = out.cpu().to(F64).view(n, H + 2 * G, hc)
+        at = 0
+        for r, a, b in rows:
+            q, k, v = want[r]
+            part = got[at:at + b - a]
+            assert (part[:, :H, :dk] - q[a:b]).abs().max() < 2e-2, ("queries", r, a)
+            assert (part[:, H:H + G, :dk] - k[a:b]).abs().max() < 2e-2, ("keys", r, a)
+            assert (part[:, H + G:, :dv] - v[a:b]).abs().max() < 2e-2 * max(1.0, float(v.abs().max())), ("values", r, a)
+            assert float(part[:, :H + G, dk:].abs().max()) == 0.0 if hc > dk else True
+            assert float(part[:, H + G:, dv:].abs().max()) == 0.0 if hc > dv else True
+            at += b - a
+            if state is not None:
+                kept = state[slots[r]].cpu().to(F64)
+                assert all(torch.equal(kept[i], data[r][b - (taps - 1) + i]) for i in range(taps - 1))
+
+
 # ------------------------------------------------------------------------------------------ the matrix memory
 def _memory_case(H, dk, dv, lens, seed, vtype=torch.float32, far=False):
     torch.manual_seed(seed)
