@@ -474,28 +474,37 @@ __global__ void mlstm_gate_values_kernel(const float* __restrict__ z, int ldz, c
   coef[(size_t)idx * 3] = log_sigmoid(cap * tanhf((row[nh + h] + (bias_f ? bias_f[h] : 0.f)) / cap));
 }
 
-// One wave a (request, head): 64 tokens at a time, each lane its token's gates; m over the 64 by a scan of the pairs
-// (F, I) that stand for m -> max(F + m, I) (first (F1, I1), then (F2, I2): (F1 + F2, max(I1 + F2, I2))).  Writes
-// coef[t, h] = (a_t, b_t, exp(-m_t)) and leaves the request's last m in its state slot at `m_at` of the head's block.
+// One wave a (request, head): 256 tokens at a time, each lane four tokens in a row.  A token's gates are the pair (F, I)
+// that stands for m -> max(F + m, I) (first (F1, I1), then (F2, I2): (F1 + F2, max(I1 + F2, I2))): a lane folds its
+// four, the wave scans the 64 results, and each lane walks its four tokens again from the maximum that the lanes
+// before it leave.  Writes coef[t, h] = (a_t, b_t, exp(-m_t)) and leaves the request's last m in its state slot at
+// `m_at` of the head's block.
 __global__ __launch_bounds__(kWave) void mlstm_gates_kernel(float* __restrict__ coef,
                                                           float* __restrict__ state, long long head_floats, long long m_at,
                                                           const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
                                                           const int32_t* __restrict__ pos0, const int32_t* __restrict__ state_slots,
                                                           int nh) {
+  constexpr int TPL = 4;   // tokens a lane
   const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int start = q_start[seq], L = q_len[seq];
   float* mp = state + ((size_t)state_slots[seq] * nh + h) * head_floats + m_at;
   float carry = pos0[seq] == 0 ? 0.f : *mp;
-  for (int base = 0; base < L; base += kWave) {
-    const int t = base + lane;
-    const bool valid = t < L;
-    float ig = -INFINITY, fg = 0.f;
-    if (valid) {
-      const float* c = coef + ((size_t)(start + t) * nh + h) * 3;
-      fg = c[0];
-      ig = c[1];
+  for (int base = 0; base < L; base += kWave * TPL) {
+    const int t0 = base + lane * TPL;
+    float fg[TPL], ig[TPL];
+    float F = 0.f, I = -INFINITY;   // the lane's tokens folded (tokens beyond the last are the identity)
+#pragma unroll
+    for (int j = 0; j < TPL; ++j) {
+      fg[j] = 0.f;
+      ig[j] = -INFINITY;
+      if (t0 + j < L) {
+        const float* c = coef + ((size_t)(start + t0 + j) * nh + h) * 3;
+        fg[j] = c[0];
+        ig[j] = c[1];
+      }
+      I = fmaxf(I + fg[j], ig[j]);
+      F += fg[j];
     }
-    float F = fg, I = ig;
 #pragma unroll
     for (int off = 1; off < kWave; off <<= 1) {
       const float Fo = __shfl_up(F, off, kWave), Io = __shfl_up(I, off, kWave);
@@ -504,14 +513,19 @@ __global__ __launch_bounds__(kWave) void mlstm_gates_kernel(float* __restrict__ 
         F = Fo + F;
       }
     }
-    const float m = fmaxf(F + carry, I);
-    float before = __shfl_up(m, 1, kWave);
-    if (lane == 0) before = carry;
-    if (valid) {
-      float* c = coef + ((size_t)(start + t) * nh + h) * 3;
-      c[0] = expf(fg + before - m);
-      c[1] = expf(ig - m);
-      c[2] = expf(-m);
+    // what the lanes before this one make of the maximum that the chunk began with
+    const float Fb = __shfl_up(F, 1, kWave), Ib = __shfl_up(I, 1, kWave);
+    float m = lane == 0 ? carry : fmaxf(Fb + carry, Ib);
+#pragma unroll
+    for (int j = 0; j < TPL; ++j) {
+      const float before = m;
+      m = fmaxf(fg[j] + before, ig[j]);
+      if (t0 + j < L) {
+        float* c = coef + ((size_t)(start + t0 + j) * nh + h) * 3;
+        c[0] = expf(fg[j] + before - m);
+        c[1] = expf(ig[j] - m);
+        c[2] = expf(-m);
+      }
     }
     carry = __shfl(m, kWave - 1, kWave);   // (lanes beyond the last token hold the identity: their m is the last token's)
   }
