@@ -82,7 +82,7 @@ def dekinex_like(shapes: dict, layers: int, window: int = 1024, experts: int = 8
     moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": experts, "top": top, "scale": 1.0}, "shared": {"ff": ff // 2}}
     attention = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "conv": 4, "scale": hd ** -0.5,
                  "rot": {"dims": hd // 2, "base": 10000.0}, "mask": {"size": window}}
-    memory = {"heads": H, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    memory = {"heads": H, "dim": hd, "vdim": hd, "gate_cap": 12.0}
     kinds = [{"type": "attention", "mixer": attention, "mlp": dense}, {"type": "mlstm", "mixer": memory, "mlp": moe},
              {"type": "attention", "mixer": attention, "mlp": moe}, {"type": "mlstm", "mixer": memory, "mlp": dense}]
     return dict(architecture="Dekinex", vocab=shapes["vocab_size"], width=d, residual_mult=0.5, norm={"eps": shapes["rms_norm_eps"]},

@@ -67,7 +67,7 @@ def test_the_pair_table_across_steps_and_slots():
 # ------------------------------------------------------------------------------------------ convolution, rotation, norm
 @pytest.mark.parametrize("H, G, dk, dv, taps, rot, dtype", [
     (4, 2, 16, 24, 4, 8, torch.float32), (3, 1, 10, 6, 3, 4, torch.float32), (2, 2, 64, 64, 2, 64, torch.bfloat16),
-    (2, 1, 136, 40, 5, 32, torch.float32), (1, 1, 32, 48, 1, 0, torch.bfloat16), (2, 2, 8, 8, 0, 2, torch.float32),
+    (2, 1, 144, 40, 5, 32, torch.float32), (1, 1, 32, 48, 1, 0, torch.bfloat16), (2, 2, 8, 8, 0, 2, torch.float32),
     (3, 3, 5, 7, 8, 2, torch.float32),
 ])
 def test_convolved_rotated_normed_heads_in_portions(H, G, dk, dv, taps, rot, dtype):
