@@ -43,6 +43,20 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// The gated unit of an EPI_SILU_MUL product, with the numbers that a clamped unit changes:
+// g' = min(g, limit), u' = clamp(u, -limit, limit), act = g' sigmoid(alpha g') (u' + plus).  As it stands here it is
+// silu(g) u to the bit.
+struct Glu {
+  float limit = INFINITY;
+  float alpha = 1.0f;
+  float plus = 0.0f;
+};
+__device__ __forceinline__ float gated_unit(float g, float u, const Glu& p) {
+  g = fminf(g, p.limit);
+  u = fminf(fmaxf(u, -p.limit), p.limit);
+  return g / (1.0f + __expf(-(p.alpha * g))) * (u + p.plus);
+}
+
 // What a product of at most 64 rows may do for the RMS norm that follows it or precedes it.
 //  * emit (the folded kernel for up to 8 rows, the skinny kernel beyond; accumulating into the float32 residual):
 //    besides the new residual r it writes h[m, n] = bf16(gamma[n] * r[m, n]), the operand of the next product, and
@@ -60,6 +74,7 @@ struct NormExtras {
   float* emit_ss;
   const float* parts;
   int n_parts;
+  Glu glu;   // the gated unit of an EPI_SILU_MUL product
 };
 
 // EPI_ROPE (the skinny kernel; the QKV product of a decode step): W stacks nh query heads, nkv key heads
@@ -112,20 +127,6 @@ constexpr int TKS = TBK / 16;           // MFMA k-steps per LDS k-step
 // tile that this launch does not need), the tile's first row and the end of its group's rows, which takes the place of M.
 // The group's W begins grp.w_stride elements a group further on; with EPI_SILU_MUL its up rows lie grp.up_off rows
 // behind its gate rows.  grp.rows, if given, names the row of A behind each row of the product.
-// The gated unit of an EPI_SILU_MUL product, with the numbers that a clamped unit changes:
-// g' = min(g, limit), u' = clamp(u, -limit, limit), act = g' sigmoid(alpha g') (u' + plus).  As it stands here it is
-// silu(g) u to the bit.
-struct Glu {
-  float limit = INFINITY;
-  float alpha = 1.0f;
-  float plus = 0.0f;
-};
-__device__ __forceinline__ float gated_unit(float g, float u, const Glu& p) {
-  g = fminf(g, p.limit);
-  u = fminf(fmaxf(u, -p.limit), p.limit);
-  return g / (1.0f + __expf(-(p.alpha * g))) * (u + p.plus);
-}
-
 struct Groups {
   const int32_t* map;
   const int32_t* rows;
@@ -1410,7 +1411,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
         for (int t = 0; t < MT; ++t) {
           const int m = t * 16 + l % 16;
           const float g = v[rt][t], u = up[(rt * MT + t) * 256 + tid + 128];
-          if (m < M && j < N / 2) c[(size_t)m * ldc + j] = (CT)(g / (1.0f + __expf(-g)) * u);
+          if (m < M && j < N / 2) c[(size_t)m * ldc + j] = (CT)gated_unit(g, u, extra.glu);
         }
       }
     }
@@ -1833,16 +1834,19 @@ extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void
 #undef GB_TL
 }
 
-// A product of many rows (more than 64) whose epilogue is the clamped gated unit (see Glu): W stacks gate rows over
-// up rows as for epilogue 2, C is bfloat16 [M, N / 2].  The kernels that serve few rows have no such form; their callers
-// apply the unit in a pass of its own.
+// A product whose epilogue is the clamped gated unit (see Glu): W stacks gate rows over up rows as for epilogue 2, C is
+// bfloat16 [M, N / 2].  Up to 64 rows the skinny kernel, beyond them the ring or the tiled kernel.
 extern "C" int gb_gemm_bf16_glu(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int M, int N, int K,
                                 float limit, float alpha, float plus, hipStream_t stream) {
-  GB_REQUIRE(M > 64 && N > 0 && N % 2 == 0 && K > 0 && K % 8 == 0, "gemm_bf16_glu: bad sizes M=%d N=%d K=%d (more than 64 rows)", M, N, K);
+  GB_REQUIRE(M > 0 && N > 0 && N % 2 == 0 && K > 0 && K % 8 == 0, "gemm_bf16_glu: bad sizes M=%d N=%d K=%d", M, N, K);
   GB_REQUIRE(ldw % 8 == 0 && lda % 8 == 0 && lda >= K && ldw >= K && ldc >= N / 2, "gemm_bf16_glu: row strides (%d, %d, %d)", lda, ldw, ldc);
   GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_bf16_glu: operands must be 16-byte aligned");
   GB_REQUIRE(limit > 0.f, "gemm_bf16_glu: the limit must be positive");
   const Glu glu{limit, alpha, plus};
+  if (M <= 64) {
+    const NormExtras extra{nullptr, 0, nullptr, 0, nullptr, nullptr, 0, glu};
+    return launch_skinny<EPI_SILU_MUL, false, bf16>(a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, nullptr, 0, 0.f, extra, stream);
+  }
   if (ring_pays(EPI_SILU_MUL, a, lda, w, ldw, M, N, K))
     return launch_ring<EPI_SILU_MUL, bf16>((const bf16*)a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, stream, glu);
   return launch_tiled<EPI_SILU_MUL, bf16>((const bf16*)a, lda, (const bf16*)w, ldw, (bf16*)c, ldc, M, N, K, stream, glu);

@@ -532,6 +532,28 @@ __global__ __launch_bounds__(kWave) void mlstm_gates_kernel(float* __restrict__ 
   if (lane == 0 && L > 0) *mp = carry;
 }
 
+// Both kernels above in one for a step in which every request brings one token: a thread a (request, head).
+__global__ void mlstm_gates_single_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ bias_i,
+                                          const float* __restrict__ bias_f, float cap, float* __restrict__ coef,
+                                          float* __restrict__ state, long long head_floats, long long m_at,
+                                          const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0,
+                                          const int32_t* __restrict__ state_slots, int n_seqs, int nh) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_seqs * nh) return;
+  const int seq = idx / nh, h = idx % nh, t = q_start[seq];
+  const float* row = z + (size_t)t * ldz;
+  const float ig = cap * tanhf((row[h] + (bias_i ? bias_i[h] : 0.f)) / cap);
+  const float fg = log_sigmoid(cap * tanhf((row[nh + h] + (bias_f ? bias_f[h] : 0.f)) / cap));
+  float* mp = state + ((size_t)state_slots[seq] * nh + h) * head_floats + m_at;
+  const float before = pos0[seq] == 0 ? 0.f : *mp;
+  const float m = fmaxf(fg + before, ig);
+  float* c = coef + ((size_t)t * nh + h) * 3;
+  c[0] = expf(fg + before - m);
+  c[1] = expf(ig - m);
+  c[2] = expf(-m);
+  *mp = m;
+}
+
 // q32 = q * q_scale, k32 = k * b_t, decay[t, h] = a_t, vext[t, h, :] = (v[t, h, :], 1): the scan's operands
 template <typename T>
 __global__ void mlstm_prep_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off,
@@ -716,16 +738,22 @@ extern "C" int gb_head_norm_gate(const float* o, const void* gate, int dtype, in
 
 // z [n, ldz] float32: the input gates' projections of the nh heads, then the forget gates'; biases float32 [nh] or nullptr;
 // coef [n, nh, 3] float32 (n: the step's rows) receives (a_t, b_t, exp(-m_t)); the running maximum of head h of a request lives at
-// state[slot][h * head_floats + m_at].
+// state[slot][h * head_floats + m_at].  single: every request of the step brings one row, and one kernel does it all.
 extern "C" int gb_mlstm_gates(const float* z, int ldz, const float* bias_i, const float* bias_f, float cap, float* coef,
                               float* state, long long head_floats, long long m_at, const int32_t* q_start,
                               const int32_t* q_len, const int32_t* pos0, const int32_t* state_slots, int n_seqs, int nh,
-                              int n, hipStream_t stream) {
+                              int n, int single, hipStream_t stream) {
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && ldz >= 2 * nh && cap > 0.f, "mlstm_gates: bad sizes requests=%d heads=%d ldz=%d cap=%g", n_seqs, nh, ldz, cap);
   GB_REQUIRE(head_floats > 0 && m_at >= 0 && m_at < head_floats, "mlstm_gates: the maximum lies outside its head's state");
   GB_REQUIRE(n_seqs <= 2147483647 && nh <= 65535, "mlstm_gates: too many heads for one launch");
   GB_REQUIRE(n >= 0 && (long long)n * nh < (1ll << 31), "mlstm_gates: too many (token, head) pairs");
   if (n_seqs == 0 || n == 0) return 0;
+  if (single) {
+    GB_REQUIRE(n == n_seqs, "mlstm_gates: a step of single tokens brings %d rows for %d requests", n, n_seqs);
+    hipLaunchKernelGGL(mlstm_gates_single_kernel, dim3((unsigned)((n_seqs * nh + 255) / 256)), dim3(256), 0, stream, z, ldz, bias_i,
+                       bias_f, cap, coef, state, head_floats, m_at, q_start, pos0, state_slots, n_seqs, nh);
+    return launched("mlstm_gates (single tokens)");
+  }
   hipLaunchKernelGGL(mlstm_gate_values_kernel, dim3((unsigned)((n * nh + 255) / 256)), dim3(256), 0, stream, z, ldz, bias_i, bias_f,
                      cap, coef, n, nh);
   hipLaunchKernelGGL(mlstm_gates_kernel, dim3(n_seqs, nh), dim3(kWave), 0, stream, coef, state, head_floats, m_at, q_start, q_len,

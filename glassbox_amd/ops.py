@@ -92,8 +92,8 @@ _SIGS = {
         "gb_linear_scan": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                            C.c_longlong, _vp],
         # z, ldz, bias_i, bias_f, cap, coef, state, floats a head, where m lies, q_start, q_len, pos0, state slots,
-        # requests, heads, rows, stream
-        "gb_mlstm_gates": [_vp, _i, _vp, _vp, _f, _vp, _vp, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+        # requests, heads, rows, every request one row (0/1), stream
+        "gb_mlstm_gates": [_vp, _i, _vp, _vp, _f, _vp, _vp, C.c_longlong, C.c_longlong, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
         # proj, dtype, stride, q_off, k_off, v_off, coef, q32, k32, decay, vext, n, heads, dk, dv, q_scale, stream
         "gb_mlstm_prep": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp],
         # o, coef, gate, dtype, gate stride, w, out, n, heads, dv, eps, stream
@@ -767,7 +767,8 @@ def mlstm_gates(z: torch.Tensor, bias_i: Optional[torch.Tensor], bias_f: Optiona
     lib = _lib("linear_attention")
     _launch(lib, lib.gb_mlstm_gates, _p(z), z.stride(0), _p(bias_i), _p(bias_f), float(cap), _p(coef), _p(state),
             int(state.shape[2] * state.shape[3]), int(m_row * state.shape[3]), _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0),
-            _p(ctx.state_slots), ctx.num_seqs, n_heads, n, _stream())
+            _p(ctx.state_slots), ctx.num_seqs, n_heads, n, 1 if int(ctx.host["max_q_len"]) == 1 and n == ctx.num_seqs else 0,
+            _stream())
 
 
 def mlstm_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, coef: torch.Tensor, q32: torch.Tensor,
@@ -1153,19 +1154,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: operand types {a.dtype} and {w.dtype} do not match a kernel")
 
 
-GLU_PRODUCT_MIN_ROWS = 65
-
-
 def gemm_glu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, limit: float, alpha: float, plus: float = 1.0) -> None:
     """out = g' * sigmoid(alpha g') * (u' + plus) with g' = min(a . gate, limit) and u' = clamp(a . up, -limit, limit),
-    formed where the product's tiles are finished: w stacks gate rows over up rows, all bfloat16, out [M, N / 2].  For
-    steps of at least ``GLU_PRODUCT_MIN_ROWS`` rows (the kernels of fewer rows have no such epilogue)."""
+    formed where the product's tiles are finished: w stacks gate rows over up rows, all bfloat16, out [M, N / 2]."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
     if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or w.shape[1] != K
-            or out.shape != (M, N // 2) or N % 2 or M < GLU_PRODUCT_MIN_ROWS):
-        raise KernelError(f"gemm_glu: bfloat16 a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match, or rows are few")
+            or out.shape != (M, N // 2) or N % 2):
+        raise KernelError(f"gemm_glu: bfloat16 a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
     lib = _lib("gemm_bf16")
     _launch(lib, lib.gb_gemm_bf16_glu, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(out), _rows(out, "out"), M, N, K,
             float(limit), float(alpha), float(plus), _stream())

@@ -104,7 +104,7 @@ class ClampedGLU(FeedForward):
     def forward(self, ctx, h, residual, store: bool = False):
         n = h.shape[0]
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
-        if ctx.dtype == torch.bfloat16 and n >= ops.GLU_PRODUCT_MIN_ROWS and ops.gemm_takes(h, self.w_gate_up):
+        if ctx.dtype == torch.bfloat16 and ops.gemm_takes(h, self.w_gate_up):
             # the unit is applied where the product's tile is finished: gate_up never reaches memory
             ops.gemm_glu(h, self.w_gate_up, act, self.limit, self.alpha)
         else:

@@ -49,16 +49,16 @@ CASES: Dict[str, dict] = {
         {"type": "attention", "mixer": {"heads": 3, "kv_heads": 1, "dim": 10, "vdim": 6, "conv": 3, "scale": 1.1,
                                         "rot": {"dims": 4, "base": 20.0}, "mask": {"size": 9}},
          "mlp": {"kind": "moe", "expert": {"ff": 12}, "router": {"experts": 5, "top": 3, "scale": 2.5}, "shared": {"ff": 7}}},
-        {"type": "mlstm", "mixer": {"heads": 2, "dim": 12, "vdim": 5, "gate_cap": 14.0}, "mlp": None},
+        {"type": "mlstm", "mixer": {"heads": 2, "dim": 12, "vdim": 5, "gate_cap": 15.0}, "mlp": None},
         {"type": "mlstm", "mixer": {"heads": 5, "dim": 6, "vdim": 10, "gate_cap": 3.0},
          "mlp": {"kind": "dense", "ff": 30, "limit": 1.5}},
     ]),
-    # a head of 144 channels (the plain attention kernel in bfloat16 too), one layer three times, five taps, a key size of
+    # a head of 136 channels (the plain attention kernel in bfloat16 too), one layer three times, five taps, a key size of
     # 128 in the matrix memory, four experts of nine
     "D": dict(architecture="Dekinex", vocab=160, width=128, residual_mult=0.25, norm={"eps": 2e-5},
               embedding={"bigram": {"buckets": 64, "mul_prev": 13, "mul_cur": 11}},
               loop={"start": 1, "stop": 2, "times": 3}, layers=[
-        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 144, "vdim": 40, "conv": 3, "scale": 0.3,
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 136, "vdim": 40, "conv": 3, "scale": 0.3,
                                         "rot": {"dims": 64, "base": 1000.0}, "mask": {"size": 50}},
          "mlp": {"kind": "dense", "ff": 72, "limit": 1.0}},
         {"type": "attention", "mixer": {"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "conv": 5, "scale": 0.4,

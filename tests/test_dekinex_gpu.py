@@ -67,7 +67,7 @@ def test_the_pair_table_across_steps_and_slots():
 # ------------------------------------------------------------------------------------------ convolution, rotation, norm
 @pytest.mark.parametrize("H, G, dk, dv, taps, rot, dtype", [
     (4, 2, 16, 24, 4, 8, torch.float32), (3, 1, 10, 6, 3, 4, torch.float32), (2, 2, 64, 64, 2, 64, torch.bfloat16),
-    (2, 1, 144, 40, 5, 32, torch.float32), (1, 1, 32, 48, 1, 0, torch.bfloat16), (2, 2, 8, 8, 0, 2, torch.float32),
+    (2, 1, 136, 40, 5, 32, torch.float32), (1, 1, 32, 48, 1, 0, torch.bfloat16), (2, 2, 8, 8, 0, 2, torch.float32),
     (3, 3, 5, 7, 8, 2, torch.float32),
 ])
 def test_convolved_rotated_normed_heads_in_portions(H, G, dk, dv, taps, rot, dtype):
@@ -238,11 +238,12 @@ def _run_memory(ops, data, rows, slots, state, H, dk, dv, cap, bias_i, bias_f, v
                                                    (5, 6, 10, 3.0, torch.float32), (2, 128, 96, 8.0, torch.float32),
                                                    (3, 8, 16, 5.0, torch.float32)])
 def test_the_matrix_memory_in_portions_of_a_batch(H, dk, dv, cap, vtype):
-    """Three requests in three steps of unequal portions, slots full of garbage: every head's normed output against the
-    plain recurrence (which the output kernel's norm leaves comparable whatever the head's size)."""
+    """Three requests in four steps of unequal portions (the last of single tokens only, which one gate kernel serves),
+    slots full of garbage: every head's normed output against the plain recurrence (which the output kernel's norm leaves
+    comparable whatever the head's size)."""
     from glassbox_amd import ops
-    lens = {0: 70, 1: 3, 2: 29}
-    cuts = {0: (1, 64, 5), 1: (1, 1, 1), 2: (27, 1, 1)}
+    lens = {0: 71, 1: 4, 2: 30}
+    cuts = {0: (1, 64, 5, 1), 1: (1, 1, 1, 1), 2: (27, 1, 1, 1)}
     slots = {0: 2, 1: 0, 2: 3}
     data = _memory_case(H, dk, dv, lens, dk * dv, vtype)
     bias_i, bias_f = torch.linspace(-1, 1, H, dtype=F64), torch.linspace(0.5, 2, H, dtype=F64)
@@ -253,7 +254,7 @@ def test_the_matrix_memory_in_portions_of_a_batch(H, dk, dv, cap, vtype):
     state = torch.full((5, H, dv + 2, dk), 77.0, device=DEV)
     done = {r: 0 for r in lens}
     tol = 3e-5 if vtype == torch.float32 else 2e-2
-    for step in range(3):
+    for step in range(4):
         rows = [(r, done[r], done[r] + cuts[r][step]) for r in lens]
         got = _run_memory(ops, data, rows, slots, state, H, dk, dv, cap, bias_i, bias_f, vtype)
         at = 0
@@ -400,10 +401,11 @@ def test_experts_on_their_own_tokens_alone(n, d, E, top, ff, sff):
     assert int(close.sum()) >= n - max(2, n // 100)
 
 
-@pytest.mark.parametrize("n, d, ff, limit", [(65, 64, 40, 0.7), (300, 96, 72, 2.0), (2048, 64, 3072, 1.0)])
+@pytest.mark.parametrize("n, d, ff, limit", [(1, 64, 40, 0.7), (8, 96, 72, 2.0), (37, 128, 1000, 1.5), (65, 64, 40, 0.7), (300, 96, 72, 2.0),
+                                            (2048, 64, 3072, 1.0)])
 def test_the_clamped_unit_where_the_products_tiles_are_finished(n, d, ff, limit):
-    """Steps of many rows apply the unit in the product's kernel (the last case in the kernel of the largest tiles); the
-    gate's sums are spread so that many lie beyond the limit on either side."""
+    """The unit is applied in the product's kernel: the kernel of few rows, the tiled one, and (the last case) the one
+    of the largest tiles; the gate's sums are spread so that many lie beyond the limit on either side."""
     from glassbox_amd import ops
     gen = torch.Generator().manual_seed(n)
     h = torch.randn(n, d, generator=gen).to(torch.bfloat16)
