@@ -576,27 +576,31 @@ __global__ void mlstm_prep_kernel(const T* __restrict__ proj, int stride, int q_
 }
 
 // out[t, h, :] = w[h, :] * y / sqrt(mean(y^2) + eps) * sigmoid(gate[t, h, :]),  y = o[t, h, :dv] / (max(|o[t, h, dv]|,
-// exp(-m_t)) + 1e-6); o holds dv + 1 sums a head, the last the normaliser's.  One wave a (token, head).
+// exp(-m_t)) + 1e-6); o holds dv + 1 sums a head, the last the normaliser's.  Sixteen lanes a (token, head), sixteen
+// heads a workgroup; a lane takes every sixteenth channel, so a head's sum is added up in one order whatever the step.
 template <typename T>
 __global__ __launch_bounds__(4 * kWave) void mlstm_out_kernel(const float* __restrict__ o, const float* __restrict__ coef,
                                                             const T* __restrict__ gate, int gate_stride,
                                                             const float* __restrict__ w, T* __restrict__ out, int nh, int dv,
                                                             float eps, int pairs) {
-  const int pair = blockIdx.x * 4 + threadIdx.x / kWave;
-  if (pair >= pairs) return;
-  const int t = pair / nh, h = pair % nh, lane = threadIdx.x % kWave;
+  constexpr int LPH = 16;   // lanes a head
+  const int pair = blockIdx.x * (4 * kWave / LPH) + threadIdx.x / LPH, li = threadIdx.x % LPH;
+  const bool live = pair < pairs;
+  const int t = live ? pair / nh : 0, h = live ? pair % nh : 0;
   const float* orow = o + ((size_t)t * nh + h) * (dv + 1);
-  const float den = fmaxf(fabsf(orow[dv]), coef[((size_t)t * nh + h) * 3 + 2]) + 1e-6f;
+  const float inv = 1.0f / (fmaxf(fabsf(orow[dv]), coef[((size_t)t * nh + h) * 3 + 2]) + 1e-6f);
   float ss = 0.f;
-  for (int d = lane; d < dv; d += kWave) {
-    const float y = orow[d] / den;
+  for (int d = li; d < dv; d += LPH) {
+    const float y = orow[d] * inv;
     ss = fmaf(y, y, ss);
   }
-  ss = wave_sum(ss);
-  const float s = 1.0f / sqrtf(ss / (float)dv + eps);
-  for (int d = lane; d < dv; d += kWave) {
+#pragma unroll
+  for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+  if (!live) return;
+  const float s = inv / sqrtf(ss / (float)dv + eps);
+  for (int d = li; d < dv; d += LPH) {
     const float g = to_f(gate[(size_t)t * gate_stride + (size_t)h * dv + d]);
-    const float y = (w ? w[(size_t)h * dv + d] : 1.0f) * ((orow[d] / den) * s);
+    const float y = (w ? w[(size_t)h * dv + d] : 1.0f) * (orow[d] * s);
     out[((size_t)t * nh + h) * dv + d] = from_f<T>(y / (1.0f + expf(-g)));
   }
 }
@@ -788,7 +792,7 @@ extern "C" int gb_mlstm_out(const float* o, const float* coef, const void* gate,
   GB_REQUIRE(n >= 0 && nh > 0 && dv > 0 && gate_stride >= nh * dv, "mlstm_out: bad sizes n=%d heads=%d dv=%d", n, nh, dv);
   GB_REQUIRE((long long)n * nh < (1ll << 31), "mlstm_out: too many (token, head) pairs");
   if (n == 0) return 0;
-  const dim3 grid((unsigned)((n * nh + 3) / 4));
+  const dim3 grid((unsigned)((n * nh + 15) / 16));
   if (dtype == kF32)
     hipLaunchKernelGGL(mlstm_out_kernel<float>, grid, dim3(4 * kWave), 0, stream, o, coef, (const float*)gate, gate_stride, w,
                        (float*)out, nh, dv, eps, n * nh);

@@ -7,8 +7,8 @@
 // `route` leaves the result in two forms: the chosen experts and their weights a token ([n, top]), and a row of E
 // weights a token with zeros for the experts not chosen (with `shared`, one more column: sigmoid of z's column E, the
 // gate of an expert that every token uses).  `gated_units` turns the stacked gate and up projections of all experts
-// into act = silu(gate) * up * weight, so that one product with the experts' down matrices side by side gives the
-// weighted sum of the chosen experts' outputs (an expert not chosen contributes exact zeros).
+// into act = silu(gate) * up * weight, so that one product with the experts' down matrices side by side adds up
+// sum_e a_e y_e over the token's experts (an expert not chosen contributes exact zeros).
 //
 // With many tokens a step, the experts run on the rows that chose them alone.  `sort` puts the (token, choice) entries
 // in the order of their experts (entries of an expert in the order of the tokens): rows[r] is the token behind sorted

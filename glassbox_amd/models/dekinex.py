@@ -1,6 +1,6 @@
 """The Dekinex decoder assembled from parts.
 
-Every layer is one norm (its weight stored around zero) whose rows feed a mixer and, where the configuration gives one,
+Every layer is one norm (the file holds its weight minus one) whose rows feed a mixer and, where the configuration gives one,
 a feed-forward; their sum, times a constant, goes into the residual (``ParallelBlock``).  The mixers: attention behind a
 short convolution (``ShortConvAttention``) and a matrix memory with exponential gates (``MLSTM``); the feed-forwards: a
 gated unit with clamped halves (``ClampedGLU``) and routed experts with a shared one (``RoutedExperts``).  A run of

@@ -193,7 +193,7 @@ class MLSTM(Mixer):
     gate i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = log sigmoid(cap tanh((W_f h + b_f) / cap)); with a
     running maximum m (0 before the first token): m_t = max(f_t + m_(t-1), i_t),
     S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T, n_t the same with k_t alone,
-    o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).  Each head's o is divided by its root mean square, the heads
+    o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).  Every head's o gets a unit-RMS norm, the heads
     side by side are multiplied by ``norm`` (a weight for every channel of every head) and by sigmoid(W_g h), and
     projected by W_o.
 

@@ -1,9 +1,9 @@
-"""A feed-forward of many small experts of which each token uses a few.
+"""A feed-forward made of many narrow gated units (experts), a few of them picked anew for every token.
 
-Router logits z = W_router h in 32-bit; scores s = sigmoid(z); the ``top`` experts with the largest s + correction are
-chosen (the correction only chooses); their weights are s / (sum of the chosen s + 1e-20) * scale.  An expert is
-W_down (silu(W_gate h) * (W_up h)) without biases, and the output is the weighted sum of the chosen experts' outputs.
-A shared expert of the same form may run for every token, times sigmoid(W_sg h), one number a token.
+z = W_router h in 32-bit and s = sigmoid(z).  A token's experts are the ``top`` largest of s + correction (the correction
+takes part in the picking alone); expert e of them gets the weight a_e = scale * s_e / (1e-20 + sum of the picked s).  An
+expert computes y_e = W_down (silu(W_gate h) * (W_up h)), no biases, and the token's result is sum_e a_e y_e.  With
+``shared_ff`` one more such unit serves all tokens, its result scaled by sigmoid(W_sg h), a scalar per token.
 
 The experts' gate matrices are stacked by rows, then their up matrices, then the shared expert's gate and up; the down
 matrices stand side by side, the shared expert's last.  A step of few tokens runs every expert on every token: one

@@ -1,5 +1,5 @@
 """RMS norm: out = g * (x / sqrt(mean(x^2) + eps)), sums in 32-bit
-(crates/glassbox-core/src/model.rs:94-100).  With ``offset`` the checkpoint stores the weight around zero and
+(crates/glassbox-core/src/model.rs:94-100).  With ``offset`` the checkpoint holds the weight minus ``offset`` and
 g = offset + w, added in 32-bit when the weights are loaded and kept in 32-bit."""
 from __future__ import annotations
 
